@@ -1,0 +1,352 @@
+"""CPU oracle for the switched mixed-precision linear path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in numpy, the arithmetic of the reference's switched linear layer so that
+the HIP kernels can be checked against it.  Only the test-suite, the smoke check and the
+benchmark's CPU-baseline leg may import it; the shipped package never does.
+
+Every function cites the reference file:line it follows (paths relative to the reference root).
+
+Pinning status (what, other than this file agreeing with itself, fixes each function):
+
+  pack_int_awq / unpack_int_awq   two independent statements of the layout in the reference
+                                  (step-by-step thirdparty/AWQ/awq_method.py:5-38, closed-form
+                                  reshape/permute test/depacking.py:8-19 and its inverse :22-38)
+                                  re-typed in tests/test_oracle_layout.py plus brute-force enumeration.
+  qfactor_layout                  closed form + width table (awq_method.py:40-75); hand cases.
+  quantize_int8 / quantize_int4   closed forms; invariants (range, reconstruction error bound).
+  dequant_to_f16 / dequant_to_i8  exact fp16 FMA rule; s=1,z=0 reduces to pure unpack; integer
+                                  zero-point reduces to textbook (q-z)*s dequantisation.
+  quant_act_i8                    hand cases (zeros, +-amax, half-way ties); the reference builds with
+                                  fast-math so its division may differ by one step on exact ties:
+                                  the specification here is IEEE fp32 division.
+  gemm_w8a8                       exact integer matmul + fixed epilogue order.
+  gemm_f16 / gemm_w4a16           parity unpinned by the reference (its fp16 GEMM is cuBLAS, its
+                                  W4A16 kernels accumulate in fp16); oracle = dequantise then fp32
+                                  accumulated matmul, tolerance 1e-2 max-abs-rel.
+  gemm_w8a16                      parity unpinned: the reference declares the id but has no
+                                  implementation (kairos/dynamic_linear.py:8-9).
+  LUT                             reference C++ header compiled into oracle/_ref (see Makefile) and
+                                  the two shipped table files.
+"""
+from __future__ import annotations
+
+import json
+import numpy as np
+
+GROUP = 128
+INTERLEAVE = 4
+KSTRIDE = 64
+
+# kairos/dynamic_linear.py:8-9 (v1) and kairos/dynamic_linear_v2.py:11-13 (v2 adds 6 and 7)
+COMP_TYPE_NAME = {
+    "w4a16_gemm": 0, "w4a16_gemv": 1, "w8a8": 2, "w8a16_gemm": 3, "w8a16_gemv": 4, "fp16": 5,
+    "w4a16_marlin": 6, "w4a8_qserve": 7,
+}
+
+
+# ----------------------------------------------------------------------------------------------
+# F: resident int4 format                                   thirdparty/AWQ/awq_method.py:5-38
+# ----------------------------------------------------------------------------------------------
+def awq_position(n, k, K):
+    """(flat int16 index, nibble) that holds element (n, k) of an [N, K] uint4 matrix.
+
+    Derived from the three permutations of awq_method.py:10-37: inside every 32-wide K block the
+    nibble is (k%32)//8; inside a 64-wide K block the four rows of a row-quad are laid side by
+    side, 16 int16 words each, and the word index inside those 16 is ((k%64)//32)*8 + k%8.
+    """
+    n = np.asarray(n, dtype=np.int64)
+    k = np.asarray(k, dtype=np.int64)
+    word = (n // 4) * K + (k // 64) * 64 + (n % 4) * 16 + ((k % 64) // 32) * 8 + (k % 8)
+    nib = (k % 32) // 8
+    return word, nib
+
+
+def pack_int_awq(q):
+    """uint4 [N, K] (any integer dtype, values 0..15) -> int16 [N/4, K]."""
+    q = np.asarray(q)
+    N, K = q.shape
+    assert N % INTERLEAVE == 0 and K % KSTRIDE == 0
+    nn, kk = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
+    word, nib = awq_position(nn, kk, K)
+    out = np.zeros(N // 4 * K, dtype=np.uint16)
+    np.bitwise_or.at(out, word.ravel(), ((q.astype(np.uint16) & 0xF) << (4 * nib).astype(np.uint16)).ravel())
+    return out.view(np.int16).reshape(N // 4, K)
+
+
+def unpack_int_awq(packed):
+    """int16 [N/4, K] -> uint8 [N, K] with values 0..15 (inverse of pack_int_awq)."""
+    packed = np.ascontiguousarray(packed)
+    N4, K = packed.shape
+    N = N4 * 4
+    flat = packed.view(np.uint16).ravel()
+    nn, kk = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
+    word, nib = awq_position(nn, kk, K)
+    return ((flat[word] >> (4 * nib).astype(np.uint16)) & 0xF).astype(np.uint8)
+
+
+# ----------------------------------------------------------------------------------------------
+# S: scale / scaled-zero tables                             thirdparty/AWQ/awq_method.py:40-75
+# ----------------------------------------------------------------------------------------------
+def calculate_zeros_width(in_features, group_size=GROUP, pack_num=8):
+    """awq_method.py:40-54: number of 8-wide column packs the [K/G] axis is padded to."""
+    if group_size >= 128:
+        mult = 1
+    elif group_size == 64:
+        mult = 2
+    elif group_size == 32:
+        mult = 4
+    else:
+        raise NotImplementedError(group_size)
+    ceil_div = lambda c, d: (c + d - 1) // d
+    return ceil_div(ceil_div(in_features // group_size, pack_num), mult) * mult
+
+
+def padded_groups(K, group_size=GROUP):
+    return calculate_zeros_width(K, group_size) * 8
+
+
+def qfactor_layout(scales, zeros, group_size=GROUP):
+    """fp16 [N, K/G] x2 -> (scales_t, scaled_zeros_t) fp16 [Gp, N]   (awq_method.py:56-75, 'kairos').
+
+    scaled_zeros = -fp16( fp32(scale_fp16) * fp32(zero) ); padded rows are zero.
+    """
+    scales = np.asarray(scales, dtype=np.float16)
+    zeros = np.asarray(zeros)
+    N, ng = scales.shape
+    Gp = padded_groups(ng * group_size, group_size)
+    qs = np.zeros((N, Gp), dtype=np.float16)
+    qs[:, :ng] = scales
+    sz = np.zeros((N, Gp), dtype=np.float16)
+    prod = qs[:, :ng].astype(np.float32) * zeros.astype(np.float32)
+    sz[:, :ng] = -(prod.astype(np.float16))
+    return np.ascontiguousarray(qs.T), np.ascontiguousarray(sz.T)
+
+
+# ----------------------------------------------------------------------------------------------
+# Q8 / Q4 / P: weight preparation
+# ----------------------------------------------------------------------------------------------
+def quantize_int8(w):
+    """kairos/quantization.py:112-141 with q_type='S', group_size=-1, max_int=127.
+
+    fp16 [N, K] -> (int8 [N, K], scale fp16 [N, 1]); all arithmetic in fp32.
+    """
+    x = np.asarray(w, dtype=np.float16).astype(np.float32)
+    amax = np.maximum(np.abs(x).max(axis=1, keepdims=True), np.float32(1e-7))
+    scale = amax / np.float32(127)
+    q = np.rint(x / scale)  # round half to even, as torch.round_
+    return q.astype(np.int8), scale.astype(np.float16)
+
+
+def quantize_int4_kairos(w8, group_size=GROUP):
+    """kairos/dynamic_linear_v2.py:15-41 (eager order; same maths as dynamic_linear.py:13-37).
+
+    int8 [N, K] -> (uint4-in-int8 [N, K], scale fp16 [N*K/G, 1], zero fp16 [N*K/G, 1]).
+    The zero-point is kept unrounded; the order of operations is x/s, + z, round, clamp.
+    """
+    w8 = np.asarray(w8)
+    shape = w8.shape
+    assert shape[-1] % group_size == 0
+    x = w8.reshape(-1, group_size).astype(np.float32)
+    mx = x.max(axis=1, keepdims=True)
+    mn = x.min(axis=1, keepdims=True)
+    scale = np.maximum(mx - mn, np.float32(1e-5)) / np.float32(15)
+    zero = -(mn / scale)
+    q = np.clip(np.rint(x / scale + zero), 0, 15)
+    with np.errstate(over="ignore"):   # a constant group makes zero overflow fp16, as in the reference
+        return q.reshape(shape).astype(np.int8), scale.astype(np.float16), zero.astype(np.float16)
+
+
+def prepare_weights(w, group_size=GROUP):
+    """kairos/dynamic_linear.py:86-115 (from_module): fp16 [N, K] -> dict of resident tensors."""
+    w = np.asarray(w, dtype=np.float16)
+    N, K = w.shape
+    w8, scale_1 = quantize_int8(w)
+    q4, scale_2, zero_2 = quantize_int4_kairos(w8, group_size)
+    scale_2 = scale_2.reshape(N, -1)
+    zero_2 = zero_2.reshape(N, -1)
+    scales_to8, scaled_zeros_to8 = qfactor_layout(scale_2, zero_2, group_size)
+    # fp16 * fp16 -> fp16 (dynamic_linear.py:108): exact product, one rounding
+    scale_f = (scale_2.astype(np.float32) * scale_1.astype(np.float32)).astype(np.float16)
+    scales, scaled_zeros = qfactor_layout(scale_f, zero_2, group_size)
+    return {
+        "qweight": pack_int_awq(q4),
+        "scales": scales, "scaled_zeros": scaled_zeros,
+        "scales_to8": scales_to8, "scaled_zeros_to8": scaled_zeros_to8,
+        "scales_1": scale_1.reshape(-1),
+        "q4": q4, "w8_step1": w8,
+    }
+
+
+# ----------------------------------------------------------------------------------------------
+# C16 / C8: on-demand conversion
+# ----------------------------------------------------------------------------------------------
+def _fma_f16(q, s, z):
+    """Single-rounding fp16 FMA: the exact value q*s+z fits in fp64, so one cast rounds once."""
+    return (q.astype(np.float64) * s.astype(np.float64) + z.astype(np.float64)).astype(np.float16)
+
+
+def _expand_groups(table, N, K, group_size):
+    """[Gp, N] table -> [N, K] by repeating each used group row group_size times."""
+    ng = K // group_size
+    return np.repeat(np.asarray(table)[:ng, :N].T, group_size, axis=1)
+
+
+def dequant_to_f16(qweight, scales, scaled_zeros, group_size=GROUP):
+    """kernels/csrc/kairos_kernel/dequant_awq_format/dequant_i4_to_f16.cu:14-36,40-151.
+
+    W16[n, k] = fma_f16(q[n, k], scales[k/G, n], scaled_zeros[k/G, n]) -> fp16 [N, K] row-major.
+    """
+    q = unpack_int_awq(qweight)
+    N, K = q.shape
+    return _fma_f16(q, _expand_groups(scales, N, K, group_size), _expand_groups(scaled_zeros, N, K, group_size))
+
+
+def dequant_to_i8(qweight, scales_to8, scaled_zeros_to8, group_size=GROUP):
+    """kernels/csrc/kairos_kernel/dequant_awq_format/dequant_i4_to_i8.cu:14-36,143-146.
+
+    W8[n, k] = (int8) fma_f16(q, s, sz): the C cast truncates toward zero.  Values outside
+    [-128, 127] cannot arise from prepare_weights(); they are clipped here.
+    """
+    f = dequant_to_f16(qweight, scales_to8, scaled_zeros_to8, group_size).astype(np.float32)
+    f = np.where(np.isnan(f), np.float32(0), f)
+    return np.clip(np.trunc(f), -128, 127).astype(np.int8)
+
+
+# ----------------------------------------------------------------------------------------------
+# A: per-token activation quantiser
+# ----------------------------------------------------------------------------------------------
+def quant_act_i8(x):
+    """kernels/csrc/kairos_kernel/quant/quant_f16_to_i8.cu:45-81 + quant/utils.cuh:77-82.
+
+    fp16 [M, K] -> (int8 [M, K], scale fp16 [M]).  amax in fp32; scale = fp16(amax/127);
+    t = 127/amax (IEEE fp32); q = sat_s8(round_half_even(fp32(x)*t)); NaN (0*inf) converts to 0.
+    """
+    xf = np.asarray(x, dtype=np.float16).astype(np.float32)
+    amax = np.abs(xf).max(axis=1, keepdims=True).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        scale = (amax / np.float32(127)).astype(np.float16)
+        t = np.float32(127) / amax
+        p = xf * t
+    p = np.where(np.isnan(p), np.float32(0), p)
+    q = np.clip(np.rint(p), -128, 127).astype(np.int8)
+    return q, scale.reshape(-1)
+
+
+# ----------------------------------------------------------------------------------------------
+# GEMMs
+# ----------------------------------------------------------------------------------------------
+def gemm_i8_acc(a8, w8):
+    """Exact int8 x int8 -> int32 accumulators, a8 [M, K], w8 [N, K] (both K-contiguous)."""
+    acc = np.asarray(a8).astype(np.float64) @ np.asarray(w8).astype(np.float64).T  # exact: |acc| < 2^53
+    return acc.astype(np.int64).astype(np.int32)
+
+
+def w8a8_epilogue(acc, wscales, ascales):
+    """thirdparty/AWQ/kernels/csrc/w8a8/w8a8_gemm_cuda.cu:889-902.
+
+    out = fp16_rn( float_rn(acc) * (float(ws[n]) * float(as[m])) ), every step rounded to fp32.
+    """
+    ws = np.asarray(wscales, dtype=np.float16).astype(np.float32).reshape(1, -1)
+    as_ = np.asarray(ascales, dtype=np.float16).astype(np.float32).reshape(-1, 1)
+    s = (ws * as_).astype(np.float32)
+    with np.errstate(over="ignore"):
+        return (acc.astype(np.float32) * s).astype(np.float32).astype(np.float16)
+
+
+def gemm_w8a8(a8, w8, wscales, ascales):
+    acc = gemm_i8_acc(a8, w8)
+    return acc, w8a8_epilogue(acc, wscales, ascales)
+
+
+def gemm_f16(x, w16):
+    """Oracle for kairos/dynamic_linear.py:163 (`input @ tmp_weight.T`): fp32 accumulation, fp16 result."""
+    with np.errstate(over="ignore"):
+        return (np.asarray(x, dtype=np.float16).astype(np.float32)
+                @ np.asarray(w16, dtype=np.float16).astype(np.float32).T).astype(np.float16)
+
+
+def gemm_w4a16(x, qweight, scales, scaled_zeros, group_size=GROUP):
+    """Oracle for gemv_forward_cuda_new / gemm_forward_cuda_new: dequantise (C16) then fp16 matmul."""
+    return gemm_f16(x, dequant_to_f16(qweight, scales, scaled_zeros, group_size))
+
+
+def gemm_w8a16(x, w8, scales_1):
+    """Build-defined W8A16: out = fp16( (x . W8^T) * scales_1[n] ), fp32 accumulation."""
+    acc = np.asarray(x, dtype=np.float16).astype(np.float32) @ np.asarray(w8).astype(np.float32).T
+    with np.errstate(over="ignore"):
+        return (acc * np.asarray(scales_1, dtype=np.float16).astype(np.float32).reshape(1, -1)).astype(np.float16)
+
+
+def switched_forward(x, prep, comp_type, bias=None):
+    """kairos/dynamic_linear.py:133-172 (_forward): x fp16 [M, K] -> fp16 [M, N] for one comp id."""
+    name = {v: k for k, v in COMP_TYPE_NAME.items()}[comp_type]
+    if name in ("w4a16_gemv", "w4a16_gemm", "fp16"):
+        out = gemm_w4a16(x, prep["qweight"], prep["scales"], prep["scaled_zeros"])
+    elif name == "w8a8":
+        w8 = dequant_to_i8(prep["qweight"], prep["scales_to8"], prep["scaled_zeros_to8"])
+        a8, sx = quant_act_i8(x)
+        out = gemm_w8a8(a8, w8, prep["scales_1"], sx)[1]
+    elif name in ("w8a16_gemm", "w8a16_gemv"):
+        w8 = dequant_to_i8(prep["qweight"], prep["scales_to8"], prep["scaled_zeros_to8"])
+        out = gemm_w8a16(x, w8, prep["scales_1"])
+    else:
+        raise ValueError(f"no oracle for comp_type {comp_type}")
+    if bias is not None:
+        out = (out.astype(np.float32) + np.asarray(bias, np.float16).astype(np.float32)).astype(np.float16)
+    return out
+
+
+def max_abs_rel(out, ref):
+    """The fp16-output tolerance metric: max|out-ref| / max|ref|."""
+    out = np.asarray(out, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.abs(out - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+# ----------------------------------------------------------------------------------------------
+# L: interval lookup table
+# ----------------------------------------------------------------------------------------------
+class LUT:
+    """kernels/csrc/kairos_kernel/lut/lut.h:8-45 semantics (the C++ variant, memo initialised to -1).
+
+    record(r, c) appends the right edge r; get(m) is c of the first segment with m <= r, and the
+    last segment's c for every m beyond the last edge.
+    """
+
+    def __init__(self):
+        self.edges = []
+        self.comps = []
+
+    def record(self, r, comp):
+        self.edges.append(int(r))
+        self.comps.append(int(comp))
+
+    def get(self, m):
+        for r, c in zip(self.edges, self.comps):
+            if m <= r:
+                return c
+        return self.comps[-1]
+
+
+def load_seg_perf_list(path):
+    """kairos/perf_profiler.py:76-81 + utils/util.py:29-30: the table file is JSON text."""
+    with open(path) as f:
+        return json.load(f)
+
+
+# ----------------------------------------------------------------------------------------------
+# synthetic inputs shared by tests and the benchmark's CPU leg
+# ----------------------------------------------------------------------------------------------
+def synth_weights(N, K, seed=10):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
+
+
+def synth_acts(M, K, seed=11, outlier_frac=0.01, outlier_gain=20.0):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    n_out = int(outlier_frac * K)
+    if n_out:
+        cols = rng.choice(K, size=n_out, replace=False)
+        x[:, cols] *= np.float32(outlier_gain)
+    return x.astype(np.float16)
