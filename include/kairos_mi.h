@@ -1,0 +1,146 @@
+/*
+ * kairos_mi.h -- C ABI of the MI355X (gfx950) switched mixed-precision linear path.
+ *
+ * Every entry point takes raw DEVICE pointers, sizes and a HIP stream (passed as void*, i.e. a
+ * hipStream_t; NULL = the null stream).  The caller owns and allocates every buffer, outputs
+ * included; nothing here allocates, frees or synchronises.  All functions are re-entrant.
+ * Return value: KMI_OK (0) or a negative KMI_E_* code; kmi_get_last_error_string() gives the
+ * calling thread's last message.  Nothing throws across this boundary.
+ *
+ * Conventions.  N = out_features, K = in_features, M = tokens, G = group size (128 only).
+ *   qweight       int16  [N/4, K]   packed uint4, four-row interleave, 64-wide K blocks
+ *                                   (thirdparty/AWQ/awq_method.py:5-38)
+ *   scales,       fp16   [Gp, N]    Gp = 8*ceil((K/G)/8) rows, row g = group g, padded rows unused
+ *   scaled_zeros                    (thirdparty/AWQ/awq_method.py:40-75); row stride is N
+ *   x / out       fp16   [M, K] / [M, N] row-major
+ *   w8 / w16      int8 / fp16 [N, K] row-major (K contiguous)
+ *   bias          fp16   [N] or NULL; added in fp16 after the product is rounded to fp16, as
+ *                 `out += bias` does (kairos/dynamic_linear.py:165-166)
+ * File:line citations name the reference interface each entry point replaces.
+ */
+#ifndef KAIROS_MI_H
+#define KAIROS_MI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KMI_OK 0
+#define KMI_E_NULL (-1)        /* a required pointer is NULL */
+#define KMI_E_SHAPE (-2)       /* a size is non-positive or violates a divisibility rule */
+#define KMI_E_GROUP (-3)       /* group size other than 128 */
+#define KMI_E_M_RANGE (-4)     /* M outside the range the kernel family supports */
+#define KMI_E_ALIGN (-5)       /* a pointer is not 16-byte aligned */
+#define KMI_E_LAUNCH (-6)      /* the HIP runtime rejected the launch */
+#define KMI_E_HANDLE (-7)      /* invalid LUT handle */
+
+#define KMI_GEMV_MAX_M 64      /* largest M kmi_gemv_w4a16 accepts */
+
+int kmi_version(void);
+const char* kmi_get_last_error_string(void);
+
+/* ---- on-demand weight conversion ------------------------------------------------------------ */
+
+/* out_f16[n,k] = fma_f16(q[n,k], scales[k/G,n], scaled_zeros[k/G,n]), single rounding.
+ * Replaces dequant_interleaved_int4_to_fp16 (kernels/csrc/pybind.cpp:22,
+ * kernels/csrc/kairos_kernel/dequant_awq_format/dequant_i4_to_f16.cu:155-185).
+ * Needs N%4==0, K%128==0. */
+int kmi_cvt_i4_to_f16(void* out_f16, const void* qweight, const void* scales, const void* scaled_zeros,
+                      int N, int K, int G, void* stream);
+
+/* out_i8[n,k] = (int8) fma_f16(q, scales_to8, scaled_zeros_to8): truncation toward zero, clipped
+ * to [-128,127].  Replaces dequant_interleaved_int4_to_int8 (kernels/csrc/pybind.cpp:23,
+ * kernels/csrc/kairos_kernel/dequant_awq_format/dequant_i4_to_i8.cu:152-180). */
+int kmi_cvt_i4_to_i8(void* out_i8, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
+                     int N, int K, int G, void* stream);
+
+/* The same two conversions, written in the tiled layout the MFMA GEMMs stage straight into LDS:
+ * [N/KMI_TILE_N][K/kb][KMI_TILE_N rows][128 bytes], kb = 64 (fp16) or 128 (int8), each row's eight
+ * 16-byte chunks XOR-swizzled by ((row>>1)&7).  No reference counterpart exists (the reference's
+ * permute_weight.cu is an uncompiled stub).  Needs N%KMI_TILE_N==0. */
+#define KMI_TILE_N 128
+int kmi_cvt_i4_to_f16_tiled(void* out_f16, const void* qweight, const void* scales, const void* scaled_zeros,
+                            int N, int K, int G, void* stream);
+int kmi_cvt_i4_to_i8_tiled(void* out_i8, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
+                           int N, int K, int G, void* stream);
+/* Inverse of the tiled layout (row-major out), for round-trip checks: elem_size 1 or 2. */
+int kmi_untile(void* out_rowmajor, const void* tiled, int N, int K, int elem_size, void* stream);
+
+/* ---- per-token activation quantiser ---------------------------------------------------------- */
+
+/* out_i8[m,k] = sat_s8(rint_half_even(float(x[m,k]) * (127.0f/amax_m))), scale[m] = fp16(amax_m/127.0f);
+ * an all-zero token gives zeros and scale 0.  Replaces quant_fp16_to_int8 (kernels/csrc/pybind.cpp:18,
+ * kernels/csrc/kairos_kernel/quant/quant_f16_to_i8.cu:86-104).  Needs K%8==0, K<=32768. */
+int kmi_quant_act_i8(void* out_i8, void* scale_f16, const void* x_f16, int M, int K, void* stream);
+
+/* ---- W4A16, small M ---------------------------------------------------------------------------- */
+
+/* out = x . dequant(qweight)^T (+bias), weights streamed once, fp32 accumulation on MFMA.
+ * Replaces gemv_forward_cuda_new (thirdparty/AWQ/kernels/csrc/pybind.cpp:23,
+ * thirdparty/AWQ/kernels/csrc/quantization_new/gemv/gemv_cuda.cu:245-463).
+ * Needs 1<=M<=KMI_GEMV_MAX_M, G==128, N%16==0, K%128==0. */
+int kmi_gemv_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
+
+/* Tuning variant: nt = 16-column tiles per wave (1,2,4), nw = waves per workgroup (4,8,16);
+ * nt<=0 or nw<=0 selects the built-in heuristic.  No reference counterpart. */
+int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                       const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                       int nt, int nw, void* stream);
+
+/* ---- MFMA GEMMs, any M ------------------------------------------------------------------------- */
+
+/* W4A16: replaces gemm_forward_cuda_new (thirdparty/AWQ/kernels/csrc/pybind.cpp:22,
+ * thirdparty/AWQ/kernels/csrc/quantization_new/gemm/gemm_cuda.cu:1126-1235); the caller supplies out. */
+int kmi_gemm_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
+
+/* W8A16: out = fp16((x . w8^T) * wscales[n]) (+bias).  The reference only declares the ids
+ * (kairos/dynamic_linear.py:8-9). */
+int kmi_gemm_w8a16(void* out_f16, const void* x_f16, const void* w8, const void* wscales_f16,
+                   const void* bias, int M, int N, int K, void* stream);
+
+/* W8A8: acc = a8 . w8^T in int32; out = fp16(float(acc) * (float(wscales[n]) * float(ascales[m]))) (+bias).
+ * Replaces w8a8_gemm_forward_cuda (thirdparty/AWQ/kernels/csrc/pybind.cpp:21,
+ * thirdparty/AWQ/kernels/csrc/w8a8/w8a8_gemm_cuda.cu:909-954). */
+int kmi_gemm_w8a8(void* out_f16, const void* a8, const void* w8, const void* wscales_f16,
+                  const void* ascales_f16, const void* bias, int M, int N, int K, void* stream);
+
+/* The same product with the raw int32 accumulators written out [M, N] (bit-exact tier). */
+int kmi_gemm_w8a8_acc_i32(void* acc_i32, const void* a8, const void* w8, int M, int N, int K, void* stream);
+
+/* FP16: out = x . w16^T (+bias), fp32 accumulation.  Replaces `input @ tmp_weight.T`
+ * (kairos/dynamic_linear.py:163). */
+int kmi_gemm_f16(void* out_f16, const void* x_f16, const void* w16, const void* bias,
+                 int M, int N, int K, void* stream);
+
+/* Variants reading the weight operand in the tiled layout written by kmi_cvt_*_tiled. */
+int kmi_gemm_w8a8_tiled(void* out_f16, const void* a8, const void* w8_tiled, const void* wscales_f16,
+                        const void* ascales_f16, const void* bias, int M, int N, int K, void* stream);
+int kmi_gemm_w8a16_tiled(void* out_f16, const void* x_f16, const void* w8_tiled, const void* wscales_f16,
+                         const void* bias, int M, int N, int K, void* stream);
+int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, const void* bias,
+                       int M, int N, int K, void* stream);
+
+/* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128 or 256. */
+void kmi_gemm_force_tile(int tile);
+
+/* ---- interval lookup table (host only) --------------------------------------------------------- */
+
+/* Replaces LUT_module.LUT (kernels/csrc/kairos_kernel/lut/lut.h:8-45, lut_bindings.cpp:5-13).
+ * record(r, c): append a segment with inclusive right edge r; get(m): c of the first segment with
+ * m <= r, the last segment's c beyond the last edge.  A one-entry memo makes repeated queries O(1);
+ * like the reference's, a table is not safe for concurrent use from several threads. */
+void* kmi_lut_new(void);
+void kmi_lut_free(void* lut);
+int kmi_lut_record(void* lut, int right_edge, int comp_type);
+int kmi_lut_get(void* lut, int m);   /* comp_type, or KMI_E_HANDLE for a NULL/empty table */
+int kmi_lut_shrink_to_fit(void* lut);
+int kmi_lut_size(void* lut);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KAIROS_MI_H */

@@ -1,0 +1,77 @@
+"""ctypes binding of libkairos_mi.so (the C ABI declared in include/kairos_mi.h).
+
+The library is the only compute path: if it is missing this module raises, nothing falls back to
+PyTorch or to the CPU.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libkairos_mi.so")
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+
+# name -> argument types (every function returns int unless listed in _RESTYPE)
+SIGNATURES = {
+    "kmi_version": [],
+    "kmi_get_last_error_string": [],
+    "kmi_cvt_i4_to_f16": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_cvt_i4_to_i8": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_cvt_i4_to_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_cvt_i4_to_i8_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_untile": [_P, _P, _I, _I, _I, _P],
+    "kmi_quant_act_i8": [_P, _P, _P, _I, _I, _P],
+    "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "kmi_gemm_w8a16": [_P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_w8a8": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_w8a8_acc_i32": [_P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_f16": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_w8a16_tiled": [_P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "kmi_gemm_force_tile": [_I],
+    "kmi_lut_new": [],
+    "kmi_lut_free": [_P],
+    "kmi_lut_record": [_P, _I, _I],
+    "kmi_lut_get": [_P, _I],
+    "kmi_lut_shrink_to_fit": [_P],
+    "kmi_lut_size": [_P],
+}
+_RESTYPE = {"kmi_get_last_error_string": ctypes.c_char_p, "kmi_lut_new": _P, "kmi_lut_free": None,
+            "kmi_gemm_force_tile": None}
+
+_lib = None
+
+
+class KairosMiError(RuntimeError):
+    """A C-ABI call returned a negative status; mirrors the RuntimeError pybind raises in the reference."""
+
+    def __init__(self, code, message):
+        super().__init__(f"[kairos_mi {code}] {message}")
+        self.code = code
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m kairos_amd.build` "
+            "(the HIP library is the only compute path; there is no fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if a declared symbol is not exported
+        fn.argtypes = args
+        fn.restype = _RESTYPE.get(name, _I)
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    if rc < 0:
+        raise KairosMiError(rc, load().kmi_get_last_error_string().decode())
+    return rc

@@ -1,0 +1,144 @@
+"""Tensor-level wrappers over the C ABI, named after the native functions of the reference that they
+replace (kernels/csrc/pybind.cpp:18-24, thirdparty/AWQ/kernels/csrc/pybind.cpp:21-23).
+
+PyTorch only supplies device memory and the current stream; every computation happens in
+libkairos_mi.so.  Outputs are allocated by the caller unless the reference function returns one.
+"""
+import torch
+
+from . import _lib
+
+GROUP_SIZE = 128
+GEMV_MAX_M = 64
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _need(t, dtype, name):
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: expected a GPU tensor (the HIP library is the only compute path)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: expected a contiguous tensor")
+    return t
+
+
+# ---- conversion ---------------------------------------------------------------------------------
+def dequant_interleaved_int4_to_fp16(output, qweight, scale, scaled_zero, group_size=GROUP_SIZE, tiled=False):
+    """output fp16 [N, K] <- packed int4 [N/4, K] (dequant_i4_to_f16.cu:155-185)."""
+    _need(output, torch.float16, "output"); _need(qweight, torch.int16, "qweight")
+    _need(scale, torch.float16, "scale"); _need(scaled_zero, torch.float16, "scaled_zero")
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    fn = _lib.load().kmi_cvt_i4_to_f16_tiled if tiled else _lib.load().kmi_cvt_i4_to_f16
+    _lib.check(fn(output.data_ptr(), qweight.data_ptr(), scale.data_ptr(), scaled_zero.data_ptr(),
+                  N, K, group_size, _stream()))
+
+
+def dequant_interleaved_int4_to_int8(output, qweight, scale, scaled_zero, group_size=GROUP_SIZE, tiled=False):
+    """output int8 [N, K] <- packed int4 [N/4, K] (dequant_i4_to_i8.cu:152-180)."""
+    _need(output, torch.int8, "output"); _need(qweight, torch.int16, "qweight")
+    _need(scale, torch.float16, "scale"); _need(scaled_zero, torch.float16, "scaled_zero")
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    fn = _lib.load().kmi_cvt_i4_to_i8_tiled if tiled else _lib.load().kmi_cvt_i4_to_i8
+    _lib.check(fn(output.data_ptr(), qweight.data_ptr(), scale.data_ptr(), scaled_zero.data_ptr(),
+                  N, K, group_size, _stream()))
+
+
+def untile(tiled, N, K):
+    """Tiled MFMA staging layout -> row-major [N, K] (verification helper)."""
+    out = torch.empty((N, K), dtype=tiled.dtype, device=tiled.device)
+    _lib.check(_lib.load().kmi_untile(out.data_ptr(), tiled.data_ptr(), N, K, tiled.element_size(), _stream()))
+    return out
+
+
+# ---- activation quantiser -----------------------------------------------------------------------
+def quant_fp16_to_int8(out, input, scale):
+    """out int8 [..., K], scale fp16 [tokens] <- input fp16 [..., K] (quant_f16_to_i8.cu:86-104)."""
+    _need(out, torch.int8, "out"); _need(input, torch.float16, "input"); _need(scale, torch.float16, "scale")
+    K = input.shape[-1]
+    M = input.numel() // K if K else 0
+    _lib.check(_lib.load().kmi_quant_act_i8(out.data_ptr(), scale.data_ptr(), input.data_ptr(), M, K, _stream()))
+
+
+# ---- products -----------------------------------------------------------------------------------
+def _flat2d(x):
+    return x.reshape(-1, x.shape[-1])
+
+
+def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZE, bias=None, cfg=None):
+    """W4A16 for small m (gemv_cuda.cu:245-463).  Returns fp16 [*x.shape[:-1], n]."""
+    _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
+    out = torch.empty(x.shape[:-1] + (n,), dtype=torch.float16, device=x.device)
+    lib = _lib.load()
+    if cfg is None:
+        rc = lib.kmi_gemv_w4a16(out.data_ptr(), x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, _stream())
+    else:
+        rc = lib.kmi_gemv_w4a16_cfg(out.data_ptr(), x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                    scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, cfg[0], cfg[1], _stream())
+    _lib.check(rc)
+    return out
+
+
+def gemm_forward(x, qweight, scales, scaled_zeros, bias=None):
+    """W4A16 MFMA GEMM for any m (gemm_cuda.cu:1126-1235).  Returns fp16 [*x.shape[:-1], N]."""
+    _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    x2 = _flat2d(x)
+    out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    _lib.check(_lib.load().kmi_gemm_w4a16(out.data_ptr(), x2.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                          scaled_zeros.data_ptr(), _ptr(bias), x2.shape[0], N, K, GROUP_SIZE, _stream()))
+    return out
+
+
+def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, tiled=False):
+    """out_feats fp16 [M, N] <- int8 [M, K] x int8 [N, K] (w8a8_gemm_cuda.cu:909-954)."""
+    _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel"); _need(out_feats, torch.float16, "out_feats")
+    M, K = in_feats.shape
+    N = out_feats.shape[-1]
+    fn = _lib.load().kmi_gemm_w8a8_tiled if tiled else _lib.load().kmi_gemm_w8a8
+    _lib.check(fn(out_feats.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), wscales.data_ptr(),
+                  ascales.data_ptr(), _ptr(bias), M, N, K, _stream()))
+
+
+def w8a8_gemm_acc_i32(in_feats, kernel, N):
+    """Raw int32 accumulators [M, N] of the W8A8 product."""
+    _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel")
+    M, K = in_feats.shape
+    acc = torch.empty((M, N), dtype=torch.int32, device=in_feats.device)
+    _lib.check(_lib.load().kmi_gemm_w8a8_acc_i32(acc.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), M, N, K, _stream()))
+    return acc
+
+
+def w8a16_gemm_forward(x, w8, wscales, N, bias=None, tiled=False):
+    """fp16 [M, N] <- fp16 [M, K] x int8 [N, K], per-channel scale in the epilogue."""
+    _need(x, torch.float16, "x"); _need(w8, torch.int8, "w8")
+    x2 = _flat2d(x)
+    M, K = x2.shape
+    out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    fn = _lib.load().kmi_gemm_w8a16_tiled if tiled else _lib.load().kmi_gemm_w8a16
+    _lib.check(fn(out.data_ptr(), x2.data_ptr(), w8.data_ptr(), wscales.data_ptr(), _ptr(bias), M, N, K, _stream()))
+    return out
+
+
+def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
+    """fp16 [M, N] <- fp16 [M, K] x fp16 [N, K] (`input @ tmp_weight.T`, dynamic_linear.py:163)."""
+    _need(x, torch.float16, "x"); _need(w16, torch.float16, "w16")
+    x2 = _flat2d(x)
+    M, K = x2.shape
+    out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    fn = _lib.load().kmi_gemm_f16_tiled if tiled else _lib.load().kmi_gemm_f16
+    _lib.check(fn(out.data_ptr(), x2.data_ptr(), w16.data_ptr(), _ptr(bias), M, N, K, _stream()))
+    return out
+
+
+def force_gemm_tile(tile):
+    """Tuning hook: 0 = automatic, else 64 / 128 / 256 (rows of the workgroup tile)."""
+    _lib.load().kmi_gemm_force_tile(int(tile))

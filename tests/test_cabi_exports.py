@@ -1,0 +1,67 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, reports argument errors without touching a GPU, and its LUT agrees with the oracle."""
+import os
+import re
+
+import pytest
+
+from oracle import kairos_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from kairos_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from kairos_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "kairos_mi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from kairos_amd import _lib
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/kairos_mi.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_argument_validation_needs_no_gpu(lib):
+    assert lib.kmi_cvt_i4_to_f16(None, None, None, None, 4, 128, 128, None) == -1
+    assert b"NULL" in lib.kmi_get_last_error_string()
+    assert lib.kmi_cvt_i4_to_i8(16, 16, 16, 16, 4, 128, 64, None) == -3
+    assert lib.kmi_cvt_i4_to_i8(16, 16, 16, 16, 6, 128, 128, None) == -2
+    assert lib.kmi_cvt_i4_to_i8(16, 8, 16, 16, 4, 128, 128, None) == -5
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 0, 64, 128, 128, None) == -4
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 65, 64, 128, 128, None) == -4
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 4, 60, 128, 128, None) == -2
+    assert lib.kmi_gemm_w8a8(16, 16, 16, 16, 16, None, 4, 64, 100, None) == -2
+    assert lib.kmi_gemm_w8a8(16, 16, 16, None, 16, None, 4, 64, 128, None) == -1
+    assert lib.kmi_quant_act_i8(16, 16, 16, 4, 12, None) == -2
+    assert lib.kmi_quant_act_i8(16, 16, 16, 0, 128, None) == 0        # empty batch is a no-op
+    assert lib.kmi_gemm_f16(16, 16, 16, None, 0, 64, 128, None) == 0
+    assert lib.kmi_lut_get(None, 3) == -7
+
+
+def test_lut_matches_oracle_on_reference_tables(lib, golden_dir):
+    for f in ("prof_llama_seg_perf_list.json", "prof_qwen_seg_perf_list.json"):
+        for seg in O.load_seg_perf_list(os.path.join(golden_dir, f)):
+            h = lib.kmi_lut_new()
+            mine = O.LUT()
+            for r, name, _ in seg:
+                lib.kmi_lut_record(h, r, O.COMP_TYPE_NAME[name])
+                mine.record(r, O.COMP_TYPE_NAME[name])
+            assert lib.kmi_lut_size(h) == len(seg)
+            lib.kmi_lut_shrink_to_fit(h)
+            for m in list(range(1, 2500)) + [5, 5, 30720, 30721, 10 ** 6, 1, 1]:
+                assert lib.kmi_lut_get(h, m) == mine.get(m)
+            lib.kmi_lut_free(h)

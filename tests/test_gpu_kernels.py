@@ -1,0 +1,306 @@
+"""GPU parity tests proper: every HIP kernel, called through the C ABI, against the CPU oracle on the
+same seeded inputs.  Bit-exact for conversion, activation quantisation and int32 accumulators;
+max-abs-rel <= 1e-2 (in practice ~1e-3) for fp16 outputs."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from oracle import kairos_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2          # fp16-output tolerance (max|out-ref| / max|ref|)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from kairos_amd import ops as _ops
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_same_bits(got, want):
+    got = np.ascontiguousarray(got)
+    want = np.ascontiguousarray(want)
+    assert got.shape == want.shape and got.dtype == want.dtype
+    bits = {1: np.uint8, 2: np.uint16, 4: np.uint32}[got.dtype.itemsize]
+    bad = np.argwhere(got.view(bits) != want.view(bits))
+    if len(bad):
+        lines = [f"{tuple(i)}: got {got[tuple(i)]!r} want {want[tuple(i)]!r}" for i in bad[:8]]
+        raise AssertionError(f"{len(bad)} of {got.size} elements differ\n" + "\n".join(lines))
+
+
+_PREP = {}
+
+
+def prep(N, K, seed=10):
+    key = (N, K, seed)
+    if key not in _PREP:
+        p = O.prepare_weights(O.synth_weights(N, K, seed))
+        p["w16"] = O.dequant_to_f16(p["qweight"], p["scales"], p["scaled_zeros"])
+        p["w8"] = O.dequant_to_i8(p["qweight"], p["scales_to8"], p["scaled_zeros_to8"])
+        _PREP[key] = p
+    return _PREP[key]
+
+
+# ------------------------------------------------------------------ conversion (C16 / C8), bit-exact
+@pytest.mark.parametrize("N,K", [(4, 128), (64, 256), (128, 512), (256, 3584), (512, 4096)])
+def test_cvt_prepared_weights_bit_exact(ops, N, K):
+    p = prep(N, K)
+    qw = dev(p["qweight"])
+    out16 = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(out16, qw, dev(p["scales"]), dev(p["scaled_zeros"]), 128)
+    assert_same_bits(host(out16), p["w16"])
+    out8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(out8, qw, dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), 128)
+    assert_same_bits(host(out8), p["w8"])
+
+
+def test_cvt_random_tables_bit_exact(ops):
+    """Arbitrary (not prepare_weights) tables: subnormal products, negative scales, saturation."""
+    N, K = 64, 512
+    rng = np.random.default_rng(21)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    qw = O.pack_int_awq(q)
+    Gp = O.padded_groups(K)
+    s = np.zeros((Gp, N), np.float16)
+    z = np.zeros((Gp, N), np.float16)
+    s[: K // 128] = rng.choice([1e-7, 3e-5, 1e-3, 0.3, 7.0, -2.5, 40.0], size=(K // 128, N)).astype(np.float16)
+    z[: K // 128] = (rng.standard_normal((K // 128, N)) * 30).astype(np.float16)
+    out16 = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(out16, dev(qw), dev(s), dev(z), 128)
+    assert_same_bits(host(out16), O.dequant_to_f16(qw, s, z))
+    out8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(out8, dev(qw), dev(s), dev(z), 128)
+    assert_same_bits(host(out8), O.dequant_to_i8(qw, s, z))
+
+
+def test_cvt_identity_is_pure_unpack(ops):
+    N, K = 128, 256
+    rng = np.random.default_rng(22)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    Gp = O.padded_groups(K)
+    out8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(out8, dev(O.pack_int_awq(q)), dev(np.ones((Gp, N), np.float16)),
+                                         dev(np.zeros((Gp, N), np.float16)), 128)
+    assert np.array_equal(host(out8), q.astype(np.int8))
+
+
+@pytest.mark.parametrize("N,K", [(128, 128), (256, 512), (384, 3584)])
+def test_cvt_tiled_roundtrip(ops, N, K):
+    p = prep(N, K)
+    qw = dev(p["qweight"])
+    t16 = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(t16, qw, dev(p["scales"]), dev(p["scaled_zeros"]), 128, tiled=True)
+    assert np.array_equal(host(ops.untile(t16, N, K)).view(np.uint16), p["w16"].view(np.uint16))
+    t8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(t8, qw, dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), 128, tiled=True)
+    assert np.array_equal(host(ops.untile(t8, N, K)), p["w8"])
+    if N * K > 128 * 128:
+        assert not np.array_equal(host(t8).reshape(N, K), p["w8"])     # the layout really is permuted
+
+
+# ------------------------------------------------------------------ activation quantiser (A), bit-exact
+@pytest.mark.parametrize("M,K", [(1, 128), (3, 4096), (16, 4096), (33, 14336), (257, 1024), (5, 28672)])
+def test_quant_act_bit_exact(ops, M, K):
+    x = O.synth_acts(M, K, seed=M + K)
+    if M >= 3:
+        x[1] = 0                                            # all-zero token
+        x[2, : min(K, 512)] = np.linspace(-3, 3, min(K, 512)).astype(np.float16)
+    q_ref, s_ref = O.quant_act_i8(x)
+    xd = dev(x)
+    q = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    s = torch.empty((M,), dtype=torch.float16, device="cuda")
+    ops.quant_fp16_to_int8(q, xd, s)
+    assert_same_bits(host(s), s_ref)
+    assert_same_bits(host(q), q_ref)
+
+
+def test_quant_act_ties_and_extremes(ops):
+    K = 128
+    x = np.zeros((4, K), np.float16)
+    x[0, :8] = [127, -127, 63.5, 62.5, 0.5, -0.5, 1.5, 2.5]
+    x[1, 0] = -65504
+    x[1, 1] = 65504
+    x[2, :3] = [6e-8, -6e-8, 0]                             # smallest subnormal
+    x[3, :4] = [2, -1, 0.5, 1e-4]
+    q_ref, s_ref = O.quant_act_i8(x)
+    q = torch.empty((4, K), dtype=torch.int8, device="cuda")
+    s = torch.empty((4,), dtype=torch.float16, device="cuda")
+    ops.quant_fp16_to_int8(q, dev(x), s)
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(s).view(np.uint16), s_ref.view(np.uint16))
+    assert host(q)[0, :8].tolist() == [127, -127, 64, 62, 0, 0, 2, 2]
+
+
+# ------------------------------------------------------------------ W4A16 small-M (Gv), 1e-2
+@pytest.mark.parametrize("M", [1, 2, 5, 16, 17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(256, 512), (1024, 4096)])
+def test_gemv_w4a16(ops, M, N, K):
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=100 + M)
+    ref = O.gemm_f16(x, p["w16"])
+    out = ops.gemv_forward(dev(x)[None], dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+    assert out.shape == (1, M, N)
+    assert O.max_abs_rel(host(out)[0], ref) < TOL
+
+
+@pytest.mark.parametrize("nt,nw", [(1, 4), (1, 8), (1, 16), (2, 4), (2, 8), (4, 4), (4, 8)])
+@pytest.mark.parametrize("M", [3, 20])
+def test_gemv_every_split(ops, M, nt, nw):
+    N, K = 512, 2048
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=7)
+    ref = O.gemm_f16(x, p["w16"])
+    out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128, cfg=(nt, nw))
+    assert O.max_abs_rel(host(out), ref) < 2e-3
+    again = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128, cfg=(nt, nw))
+    assert torch.equal(out, again)                          # fixed reduction order
+
+
+def test_gemv_bias_and_ragged_strip(ops):
+    N, K, M = 48, 256, 4                                    # N is not a multiple of the 64-column strip
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=3)
+    bias = (np.random.default_rng(1).standard_normal(N)).astype(np.float16)
+    ref = (O.gemm_f16(x, p["w16"]).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128,
+                           bias=dev(bias), cfg=(4, 4))
+    assert O.max_abs_rel(host(out), ref) < 2e-3
+
+
+# ------------------------------------------------------------------ MFMA GEMMs
+GEMM_M = [1, 7, 64, 65, 130, 300]
+
+
+@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("M", GEMM_M)
+def test_gemm_w8a8_int32_bit_exact(ops, M, tile):
+    N, K = 384, 1024
+    rng = np.random.default_rng(M)
+    a8 = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    w8 = rng.integers(-128, 128, size=(N, K)).astype(np.int8)
+    ops.force_gemm_tile(tile)
+    try:
+        acc = ops.w8a8_gemm_acc_i32(dev(a8), dev(w8), N)
+    finally:
+        ops.force_gemm_tile(0)
+    assert np.array_equal(host(acc), O.gemm_i8_acc(a8, w8))
+
+
+def test_gemm_w8a8_extreme_accumulator(ops):
+    M, N, K = 2, 128, 14336
+    a8 = np.full((M, K), -128, np.int8)
+    w8 = np.full((N, K), -128, np.int8)
+    acc = host(ops.w8a8_gemm_acc_i32(dev(a8), dev(w8), N))
+    assert (acc == 128 * 128 * K).all()
+
+
+@pytest.mark.parametrize("tile", [0, 64, 128, 256])
+@pytest.mark.parametrize("M", GEMM_M)
+def test_gemm_w8a8_path(ops, M, tile):
+    """The whole w8a8 lane: C8 -> A -> G8, against the oracle lane; the fp16 result is compared bit for bit
+    because the epilogue order is fixed."""
+    N, K = 256, 512
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=200 + M)
+    ref = O.switched_forward(x, p, O.COMP_TYPE_NAME["w8a8"])
+    w8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(w8, dev(p["qweight"]), dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), 128)
+    xd = dev(x)
+    a8 = torch.empty_like(xd, dtype=torch.int8)
+    sx = torch.empty((M,), dtype=torch.float16, device="cuda")
+    ops.quant_fp16_to_int8(a8, xd, sx)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.force_gemm_tile(tile)
+    try:
+        ops.w8a8_gemm_forward(a8, w8, dev(p["scales_1"]), sx, out)
+    finally:
+        ops.force_gemm_tile(0)
+    assert_same_bits(host(out), ref)
+
+
+@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("M", GEMM_M)
+def test_gemm_w4a16_f16_w8a16(ops, M, tile):
+    N, K = 384, 1024
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=300 + M)
+    ref = O.gemm_f16(x, p["w16"])
+    xd = dev(x)
+    ops.force_gemm_tile(tile)
+    try:
+        out4 = ops.gemm_forward(xd, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]))
+        out16 = ops.f16_gemm_forward(xd, dev(p["w16"]), N)
+        out816 = ops.w8a16_gemm_forward(xd, dev(p["w8"]), dev(p["scales_1"]), N)
+    finally:
+        ops.force_gemm_tile(0)
+    assert O.max_abs_rel(host(out4), ref) < 2e-3
+    assert O.max_abs_rel(host(out16), ref) < 2e-3
+    assert torch.equal(out4, out16)                         # same fp16 weights, same accumulation order
+    assert O.max_abs_rel(host(out816), O.gemm_w8a16(x, p["w8"], p["scales_1"])) < 2e-3
+
+
+@pytest.mark.parametrize("tile", [64, 128, 256])
+def test_gemm_tiled_operands_match_row_major(ops, tile):
+    N, K, M = 384, 1024, 150
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=5)
+    xd = dev(x)
+    qw = dev(p["qweight"])
+    t16 = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(t16, qw, dev(p["scales"]), dev(p["scaled_zeros"]), 128, tiled=True)
+    t8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(t8, qw, dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), 128, tiled=True)
+    a8 = torch.empty_like(xd, dtype=torch.int8)
+    sx = torch.empty((M,), dtype=torch.float16, device="cuda")
+    ops.quant_fp16_to_int8(a8, xd, sx)
+    s1 = dev(p["scales_1"])
+    ops.force_gemm_tile(tile)
+    try:
+        a = ops.f16_gemm_forward(xd, dev(p["w16"]), N)
+        b = ops.f16_gemm_forward(xd, t16, N, tiled=True)
+        c = ops.w8a16_gemm_forward(xd, dev(p["w8"]), s1, N)
+        d = ops.w8a16_gemm_forward(xd, t8, s1, N, tiled=True)
+        e = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        f = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        ops.w8a8_gemm_forward(a8, dev(p["w8"]), s1, sx, e)
+        ops.w8a8_gemm_forward(a8, t8, s1, sx, f, tiled=True)
+    finally:
+        ops.force_gemm_tile(0)
+    assert torch.equal(a, b) and torch.equal(c, d) and torch.equal(e, f)
+
+
+def test_gemm_bias(ops):
+    N, K, M = 256, 512, 33
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=8)
+    bias = np.random.default_rng(2).standard_normal(N).astype(np.float16)
+    ref = O.switched_forward(x, p, O.COMP_TYPE_NAME["fp16"], bias=bias)
+    out = ops.gemm_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), bias=dev(bias))
+    assert O.max_abs_rel(host(out), ref) < 2e-3
+
+
+# ------------------------------------------------------------------ error behaviour of the boundary
+def test_argument_errors(ops):
+    from kairos_amd import _lib
+    N, K = 64, 256
+    p = prep(N, K)
+    x = dev(O.synth_acts(4, K))
+    with pytest.raises(_lib.KairosMiError) as e:
+        ops.gemv_forward(x, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), 4, N, K, 64)
+    assert e.value.code == -3
+    big = dev(O.synth_acts(65, K))
+    with pytest.raises(_lib.KairosMiError) as e:
+        ops.gemv_forward(big, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), 65, N, K, 128)
+    assert e.value.code == -4
+    with pytest.raises(TypeError):
+        ops.quant_fp16_to_int8(torch.empty((4, K), dtype=torch.int8, device="cuda"), x.float(), torch.empty(4, dtype=torch.float16, device="cuda"))
