@@ -1,0 +1,329 @@
+#!/usr/bin/env python3
+"""Benchmark of the LUT-switched mixed-precision linear path on one MI355X.
+
+Workload (BASELINE.json configs[1]): the four linear shapes of one Llama-3-8B decoder layer
+(qkv 4096->6144, o_proj 4096->4096, gate_up 4096->28672, down 14336->4096), M in {1,2,4,...,4096}.
+One STEP = for every M of the grid, one decoder layer's four linears through DynamicLinear.forward
+(LUT lookup -> selected HIP lane, conversion and activation quantisation included).  Weights are
+synthetic N(0, 0.02) fp16 quantised by the module's own from_module; activations N(0,1) with 1 % of
+the K channels scaled x20.  Several copies of the layer are rotated so that consecutive calls do not
+find their weights in the 256 MB Infinity Cache.
+
+Prints ONE JSON line.  `value` = microseconds per layer (four linears) averaged over the M grid.
+`roofline` describes the kernel that takes the most time in a step, timed with device events on the
+launch stream in an instrumented replay of the same steps.  `cpu_baseline` times the numpy oracle.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LAYER = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)]
+M_GRID = [1 << i for i in range(13)]
+PEAK = {"hbm": 8.0e12, "f16": 2.5e15, "i8": 5.0e15}       # MI355X published: HBM3E B/s, dense MFMA op/s
+LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x")
+G = 128
+
+
+def algorithmic(kernel, M, N, K):
+    """(bytes, flops, mfma dtype or None) per launch -- the per-unit figures of the scope table."""
+    if kernel in ("gemv_w4a16", "gemm_w4a16"):
+        return N * K // 2 + 2 * (K // G) * N * 2 + M * K * 2 + M * N * 2, 2 * M * N * K, "f16"
+    if kernel == "cvt_i4_to_i8":
+        return N * K // 2 + 4 * (K // G) * N + N * K, 0, None
+    if kernel == "cvt_i4_to_f16":
+        return N * K // 2 + 4 * (K // G) * N + 2 * N * K, 0, None
+    if kernel == "quant_act_i8":
+        return M * K * 2 + M * K + 2 * M, 0, None
+    if kernel == "gemm_w8a8":
+        return M * K + N * K + 2 * N + 2 * M + 2 * M * N, 2 * M * N * K, "i8"
+    if kernel == "gemm_w8a16":
+        return 2 * M * K + N * K + 2 * N + 2 * M * N, 2 * M * N * K, "f16"
+    if kernel == "gemm_f16":
+        return 2 * M * K + 2 * N * K + 2 * M * N, 2 * M * N * K, "f16"
+    raise KeyError(kernel)
+
+
+def roofline_time(kernel, M, N, K):
+    b, f, dt = algorithmic(kernel, M, N, K)
+    t_mem = b / PEAK["hbm"]
+    t_cmp = f / PEAK[dt] if dt else 0.0
+    return max(t_mem, t_cmp), ("hbm" if t_mem >= t_cmp else "mfma")
+
+
+class Tracer:
+    """Brackets every kernel launch with a pair of device events on the launch stream."""
+
+    def __init__(self, torch, ops):
+        self.torch, self.ops = torch, ops
+        self.records = []          # (label, kernel, M, N, K, start_event, end_event)
+        self._cur = None
+
+    def begin(self, name, M, N, K):
+        label = name
+        if name.startswith("gemm_"):
+            label = f"{name}[{self.ops.gemm_tile_for(M, N)}]"
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self._cur = (label, name, M, N, K, ev)
+
+    def end(self):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.records.append(self._cur + (ev,))
+
+    def summarise(self):
+        self.torch.cuda.synchronize()
+        agg = {}
+        for label, name, M, N, K, e0, e1 in self.records:
+            a = agg.setdefault(label, {"kernel": name, "launches": 0, "sec": 0.0, "bytes": 0, "flops": 0, "dt": None,
+                                       "ideal_sec": 0.0})
+            b, f, dt = algorithmic(name, M, N, K)
+            a["launches"] += 1
+            a["sec"] += e0.elapsed_time(e1) * 1e-3
+            a["bytes"] += b
+            a["flops"] += f
+            a["dt"] = dt
+            a["ideal_sec"] += roofline_time(name, M, N, K)[0]
+        return agg
+
+
+def cpu_baseline(gpu_us_same_sample):
+    """Oracle lane (dequantise + fp32-accumulated matmul) on config 1, one thread."""
+    import numpy as np
+    from oracle import kairos_oracle as O
+    try:
+        from threadpoolctl import threadpool_limits
+    except ImportError:                                      # pragma: no cover
+        threadpool_limits = None
+    N = K = 4096
+    M = 16
+    prep = O.prepare_weights(O.synth_weights(N, K))
+    x = O.synth_acts(M, K)
+
+    def once():
+        t0 = time.perf_counter()
+        O.gemm_w4a16(x, prep["qweight"], prep["scales"], prep["scaled_zeros"])
+        return time.perf_counter() - t0
+
+    ctx = threadpool_limits(limits=1) if threadpool_limits else None
+    if ctx:
+        ctx.__enter__()
+    try:
+        once()
+        ts = sorted(once() for _ in range(7))
+    finally:
+        if ctx:
+            ctx.__exit__(None, None, None)
+    med = ts[len(ts) // 2]
+    layer_weights = sum(n * k for _, n, k in LAYER)
+    scale = layer_weights / (N * K)
+    return {"value": med * 1e6 * scale, "unit": "us/layer at M=16 (W4A16 lane)", "cores": 1, "kind": "port",
+            "sample": f"numpy oracle, dequantise + matmul of one 4096x4096 linear at M=16 (median of 7: {med * 1e3:.1f} ms), "
+                      f"scaled by the layer's weight count (x{scale:.2f}); the GPU spends {gpu_us_same_sample:.1f} us on the same linear"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--copies", type=int, default=4, help="layer copies rotated to defeat the Infinity Cache")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-lane sweep table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is single-GPU by construction (every linear is independent; see the sharding note "
+              "in DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP library is the only compute path", file=sys.stderr)
+        sys.exit(3)
+    from kairos_amd import ops
+    from kairos_amd.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos_amd.perf_profiler import Profiler
+    from kairos_amd.weight_prep import prepare_linear_weight
+    from oracle import kairos_oracle as O                     # synthetic inputs + the CPU leg only
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    names = {v: k for k, v in COMP_TYPE_NAME.items()}
+
+    # ---- synthetic layer copies --------------------------------------------------------------
+    layers = []
+    for _name, N, K in LAYER:
+        w = torch.from_numpy(O.synth_weights(N, K, seed=10)).to(dev)
+        prep = prepare_linear_weight(w)
+        del w
+        copies = []
+        for c in range(args.copies):
+            dl = DynamicLinear(K, N, False, dev, 128)
+            for key, val in prep.items():
+                setattr(dl, key, val if c == 0 else val.clone())
+            copies.append(dl)
+        layers.append(copies)
+    acts = {}
+    for K in sorted({k for _, _, k in LAYER}):
+        for M in M_GRID:
+            acts[(M, K)] = torch.from_numpy(O.synth_acts(M, K, seed=11)).to(dev).reshape(1, M, K)
+
+    # ---- lookup table -------------------------------------------------------------------------
+    shapes = [(N, K) for _, N, K in LAYER]
+    prof = Profiler(shapes)
+    lut_source = "committed MI355X table"
+    if os.path.exists(os.path.join(LUT_DIR, "seg_perf_list.pt")):
+        prof.load(LUT_DIR + "/")
+    else:
+        lut_source = "profiled at start-up (n=20)"
+        prof.profiling(input_len=M_GRID, n=20, preheat_time=5)
+    DynamicLinear.prof = prof
+
+    def step(s):
+        for mi, M in enumerate(M_GRID):
+            c = (s * len(M_GRID) + mi) % args.copies
+            for li, (_n, _N, K) in enumerate(LAYER):
+                layers[li][c](acts[(M, K)])
+
+    # ---- timed region -------------------------------------------------------------------------
+    for s in range(args.warmup):
+        step(s)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for s in range(args.steps):
+        step(s)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    us_per_layer = ms_per_step * 1e3 / len(M_GRID)
+
+    # ---- instrumented replay of the same steps: per-kernel device time ---------------------------
+    tracer = Tracer(torch, ops)
+    ops.set_tracer(tracer)
+    try:
+        for s in range(args.steps):
+            step(s)
+    finally:
+        ops.set_tracer(None)
+    agg = tracer.summarise()
+    total_kernel_sec = sum(a["sec"] for a in agg.values())
+    dom_label, dom = max(agg.items(), key=lambda kv: kv[1]["sec"])
+    conv_sec = sum(a["sec"] for a in agg.values() if a["kernel"].startswith("cvt_"))
+    avg_dur = dom["sec"] / dom["launches"]
+    t_mem = dom["bytes"] / PEAK["hbm"]
+    t_cmp = dom["flops"] / PEAK[dom["dt"]] if dom["dt"] else 0.0
+    if t_cmp > t_mem:
+        achieved, peak, unit, bound = dom["flops"] / dom["sec"] / 1e12, PEAK[dom["dt"]] / 1e12, "TFLOP/s", "mfma"
+    else:
+        achieved, peak, unit, bound = dom["bytes"] / dom["sec"] / 1e9, PEAK["hbm"] / 1e9, "GB/s", "hbm"
+    roofline = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                "frac": round(achieved / peak, 4), "traffic": None, "kernel": dom_label,
+                "launches": dom["launches"], "avg_launch_us": round(avg_dur * 1e6, 2),
+                "share_of_kernel_time": round(dom["sec"] / total_kernel_sec, 4)}
+    kernels = {k: {"launches": a["launches"], "avg_us": round(a["sec"] / a["launches"] * 1e6, 2),
+                   "share": round(a["sec"] / total_kernel_sec, 4),
+                   "roofline_frac": round(a["ideal_sec"] / a["sec"], 4)} for k, a in sorted(agg.items())}
+
+    # ---- per-M view of the switched path and per-lane sweep ---------------------------------------
+    def time_calls(fn, n):
+        fn(); fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(n):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n             # us
+
+    by_m = {}
+    for M in M_GRID:
+        n = 30 if M <= 512 else 10
+
+        def layer_call(i=0, M=M):
+            for li, (_n, _N, K) in enumerate(LAYER):
+                layers[li][i % args.copies](acts[(M, K)])
+        by_m[M] = round(time_calls(layer_call, n), 2)
+
+    sweep = []
+    if not args.no_sweep:
+        lanes = ["w4a16_gemv", "w4a16_gemm", "w8a16_gemm", "w8a8", "fp16"]
+        for li, (lname, N, K) in enumerate(LAYER):
+            for M in M_GRID:
+                for lane in lanes:
+                    if lane == "w4a16_gemv" and M > ops.GEMV_MAX_M:
+                        continue
+                    cid = COMP_TYPE_NAME[lane]
+                    n = 20 if M <= 512 else 6
+
+                    def call(i=0, cid=cid, M=M, K=K, li=li):
+                        layers[li][i % args.copies]._forward(acts[(M, K)], M, cid)
+                    us = time_calls(call, n)
+                    main_kernel = {"w4a16_gemv": "gemv_w4a16", "w4a16_gemm": "gemm_w4a16", "w8a16_gemm": "gemm_w8a16",
+                                   "w8a8": "gemm_w8a8", "fp16": "gemm_f16"}[lane]
+                    ideal, bnd = roofline_time(main_kernel, M, N, K)
+                    b, f, _dt = algorithmic(main_kernel, M, N, K)
+                    sweep.append({"shape": lname, "N": N, "K": K, "M": M, "lane": lane, "us": round(us, 2),
+                                  "tflops": round(f / us / 1e6, 2), "gbps": round(b / us / 1e3, 1), "bound": bnd,
+                                  "roofline_frac": round(ideal * 1e6 / us, 4),
+                                  "lut_pick": names[prof.get_comp_type((N, K), M)] == lane})
+        out = args.out or os.path.join(ROOT, "gpurun_out", "bench_sweep.json")
+        try:
+            os.makedirs(os.path.dirname(out), exist_ok=True)
+            with open(out, "w") as fh:
+                json.dump({"sweep": sweep, "by_m_us_per_layer": by_m, "kernels": kernels}, fh, indent=1)
+        except OSError:
+            pass
+        print(f"{'shape':8s} {'M':>5s} " + " ".join(f"{l:>18s}" for l in lanes), file=sys.stderr)
+        for lname, N, K in LAYER:
+            for M in M_GRID:
+                cells = []
+                for lane in lanes:
+                    r = [s for s in sweep if s["shape"] == lname and s["M"] == M and s["lane"] == lane]
+                    cells.append(f"{r[0]['us']:9.1f}us {100 * r[0]['roofline_frac']:5.1f}%{'*' if r[0]['lut_pick'] else ' '}"
+                                 if r else " " * 18)
+                print(f"{lname:8s} {M:5d} " + " ".join(cells), file=sys.stderr)
+
+    # best roofline fractions in the two regimes the targets name
+    def best(pred):
+        rows = [s for s in sweep if pred(s)]
+        return max(rows, key=lambda s: s["roofline_frac"]) if rows else None
+    small = best(lambda s: s["M"] <= 16 and s["lane"] == "w4a16_gemv")
+    large = best(lambda s: s["M"] >= 1024 and s["lane"] in ("w8a8", "w4a16_gemm", "fp16", "w8a16_gemm"))
+
+    # the GPU on the CPU leg's sample: config 1 through the small-M lane
+    cfg1_us = time_calls(lambda i=0: layers[1][i % args.copies]._forward(acts[(16, 4096)], 16, COMP_TYPE_NAME["w4a16_gemv"]), 50)
+    cpu = None if args.no_cpu else cpu_baseline(cfg1_us)
+
+    result = {
+        "metric": "switched mpGEMM us/layer over M=1..4096, Llama-3-8B shapes",
+        "value": round(us_per_layer, 2), "unit": "us/layer (mean over the 13-point M grid)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16+i8 (LUT-switched: fp16 MFMA / int8 MFMA lanes, fp32 / int32 accumulation)", "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3-8B linear-shape sweep, qkv 4096->6144, o_proj 4096->4096, "
+                               "gate_up 4096->28672, down 14336->4096; M in {1,2,4,...,4096}; LUT-switched DynamicLinear.forward",
+                   "group_size": 128, "layer_copies_rotated": args.copies, "lut": lut_source,
+                   "lut_segments": prof.seg_perf_list},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "wall_s_timed_region": round(wall, 3),
+        "conversion_share_of_kernel_time": round(conv_sec / total_kernel_sec, 4),
+        "kernels": kernels, "us_per_layer_by_m": by_m,
+        "best_small_m": small and {k: small[k] for k in ("shape", "M", "us", "gbps", "roofline_frac")},
+        "best_large_m": large and {k: large[k] for k in ("shape", "M", "lane", "us", "tflops", "roofline_frac")},
+        "config1_gemv_us": round(cfg1_us, 2),
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -126,6 +126,8 @@ int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, 
 
 /* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128 or 256. */
 void kmi_gemm_force_tile(int tile);
+/* The workgroup tile (64, 128 or 256 rows) the automatic choice uses for an M x N output. */
+int kmi_gemm_pick_tile(int M, int N);
 
 /* ---- interval lookup table (host only) --------------------------------------------------------- */
 

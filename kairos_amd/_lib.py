@@ -33,6 +33,7 @@ SIGNATURES = {
     "kmi_gemm_w8a16_tiled": [_P, _P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_force_tile": [_I],
+    "kmi_gemm_pick_tile": [_I, _I],
     "kmi_lut_new": [],
     "kmi_lut_free": [_P],
     "kmi_lut_record": [_P, _I, _I],

@@ -274,15 +274,17 @@ static int launch_gemm(const GemmArgs& a, hipStream_t st) {
 }
 
 // Tile choice: the largest tile that still yields about one workgroup per CU.
+static int pick_tile(int M, int N) {
+    auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    if (M > 128 && wgs(256, 256) >= 200) return 256;
+    if (M > 64 && wgs(128, 128) >= 128) return 128;
+    return 64;
+}
+extern "C" int kmi_gemm_pick_tile(int M, int N) { return pick_tile(M, N); }
+
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
-    auto wgs = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-    int tile = force_tile;
-    if (tile <= 0) {
-        if (a.M > 128 && wgs(256, 256) >= 200) tile = 256;
-        else if (a.M > 64 && wgs(128, 128) >= 128) tile = 128;
-        else tile = 64;
-    }
+    const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N);
     switch (tile) {
         case 256: return launch_gemm<KIND, 256, 256, TILED>(a, st);
         case 128: return launch_gemm<KIND, 128, 128, TILED>(a, st);

@@ -1,0 +1,134 @@
+"""DynamicLinear: the LUT-switched mixed-precision linear layer (kairos/dynamic_linear.py:39-175).
+
+Weights are resident only as packed int4 (+ fp16 scale tables).  Each call looks M = tokens up in
+the offline-profiled interval table of this layer's shape and runs one of the HIP kernel lanes:
+
+    w4a16_gemv (1)  small-M MFMA streaming kernel            kmi_gemv_w4a16
+    w4a16_gemm (0)  LDS-staged MFMA GEMM, int4 decoded on the fly   kmi_gemm_w4a16
+    w8a8       (2)  int4->int8 conversion + per-token int8 activations + int8 MFMA GEMM
+    w8a16_*  (3,4)  int4->int8 conversion + fp16 activations, fp16 MFMA GEMM (declared but unused upstream)
+    fp16       (5)  int4->fp16 conversion + fp16 MFMA GEMM
+
+Same constructor, class attribute `prof`, `from_module`, `forward`, `_forward` and tensor attributes
+as the reference module.
+"""
+import itertools
+
+import torch
+
+from . import ops
+from .temp_cache import default_cache
+from .weight_prep import prepare_linear_weight
+
+COMP_TYPE_NAME = {'w4a16_gemm': 0, 'w4a16_gemv': 1, 'w8a8': 2,
+                  'w8a16_gemm': 3, 'w8a16_gemv': 4, 'fp16': 5}
+
+_W4A16_GEMM, _W4A16_GEMV, _W8A8, _W8A16_GEMM, _W8A16_GEMV, _FP16 = 0, 1, 2, 3, 4, 5
+_uids = itertools.count(1)
+
+
+class DynamicLinear(torch.nn.Module):
+    prof = None                 # Profiler shared by every instance, set by the caller (kairos/main.py:52)
+    tiled_weights = True        # converted weights are written in the tiled MFMA staging layout
+    temp_cache = None           # None -> the process-wide default cache
+
+    @torch.no_grad()
+    def __init__(self, in_features, out_features, bias, device, group_size):
+        super().__init__()
+        self.enable_accel = False
+        self.return_dtype = torch.float16
+        self.in_features = in_features
+        self.out_features = out_features
+        self.group_size = group_size
+        if bias:
+            self.register_buffer("bias", torch.empty((out_features,), device=device, dtype=torch.float16))
+        else:
+            self.bias = None
+        self.shape = (out_features, in_features)
+        self.pre_m = 0
+        self.pre_comp_type = ''
+        self.comp_type = None
+        self._uid = next(_uids)     # identifies this layer's entries in the temp cache
+        self.switch_count = 0       # times the selected lane changed between consecutive forward calls
+        self.qweight = self.scales = self.scaled_zeros = None
+        self.scales_to8 = self.scaled_zeros_to8 = self.scales_1 = None
+
+    @classmethod
+    @torch.no_grad()
+    def from_module(cls, linear, device, return_dtype=torch.float16, init_only=False, name=''):
+        q_linear = cls(linear.in_features, linear.out_features, linear.bias is not None, device, group_size=128)
+        if init_only:
+            return q_linear
+        prepared = prepare_linear_weight(linear.weight.data, group_size=128)
+        for key, value in prepared.items():
+            setattr(q_linear, key, value.to(device))
+        if linear.bias is not None:
+            q_linear.bias = linear.bias.detach().clone().half().to(device)
+        return q_linear
+
+    # ------------------------------------------------------------------------------------------
+    def _cache(self):
+        return self.temp_cache if self.temp_cache is not None else default_cache()
+
+    def _tileable(self):
+        return self.tiled_weights and self.out_features % 128 == 0
+
+    def _converted(self, fmt):
+        """int8 or fp16 copy of the weight in the temp cache; converts only if it is not there."""
+        tiled = self._tileable()
+        dtype = torch.int8 if fmt == 'i8' else torch.float16
+        buf, hit = self._cache().get(self._uid, (fmt, tiled), self.shape, dtype, self.qweight.device)
+        if not hit:
+            if fmt == 'i8':
+                ops.dequant_interleaved_int4_to_int8(buf, self.qweight, self.scales_to8, self.scaled_zeros_to8,
+                                                     self.group_size, tiled=tiled)
+            else:
+                ops.dequant_interleaved_int4_to_fp16(buf, self.qweight, self.scales, self.scaled_zeros,
+                                                     self.group_size, tiled=tiled)
+        return buf, tiled
+
+    @torch.no_grad()
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        shape = input.shape
+        input = input.reshape(-1, shape[-1])
+        m = input.shape[0]
+        if m != self.pre_m:
+            self.pre_m = m
+            comp = type(self).prof.get_comp_type(self.shape, m)
+            if self.comp_type is not None and comp != self.comp_type:
+                self.switch_count += 1
+            self.comp_type = comp
+        return self._forward(input, m, self.comp_type).reshape(*shape[:-1], -1)
+
+    @torch.no_grad()
+    def _forward(self, input: torch.Tensor, batch_token_len, comp_type) -> torch.Tensor:
+        N, K = self.shape
+        lead = input.shape[:-1]
+        x = input.reshape(-1, K)
+        if not x.is_contiguous():
+            x = x.contiguous()
+        m = x.shape[0]
+        if comp_type == _W4A16_GEMV and m <= ops.GEMV_MAX_M:
+            out = ops.gemv_forward(x, self.qweight, self.scales, self.scaled_zeros, m, N, K,
+                                   self.group_size, bias=self.bias)
+        elif comp_type in (_W4A16_GEMM, _W4A16_GEMV):
+            out = ops.gemm_forward(x, self.qweight, self.scales, self.scaled_zeros, bias=self.bias)
+        elif comp_type == _W8A8:
+            w8, tiled = self._converted('i8')
+            int_x = torch.empty_like(x, dtype=torch.int8)
+            scale_x = torch.empty((m,), device=x.device, dtype=torch.float16)
+            ops.quant_fp16_to_int8(int_x, x, scale_x)
+            out = torch.empty((m, N), device=x.device, dtype=torch.float16)
+            ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
+        elif comp_type in (_W8A16_GEMM, _W8A16_GEMV):
+            w8, tiled = self._converted('i8')
+            out = ops.w8a16_gemm_forward(x, w8, self.scales_1, N, bias=self.bias, tiled=tiled)
+        elif comp_type == _FP16:
+            w16, tiled = self._converted('f16')
+            out = ops.f16_gemm_forward(x, w16, N, bias=self.bias, tiled=tiled)
+        else:
+            raise ValueError(f"unknown comp_type id {comp_type}")
+        return out.reshape(*lead, N)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"

@@ -11,6 +11,25 @@ from . import _lib
 GROUP_SIZE = 128
 GEMV_MAX_M = 64
 
+# Optional kernel tracer (profiling tools): an object with begin(name, M, N, K) / end() that is
+# called around every kernel launch.  None in normal operation.
+_tracer = None
+
+
+def set_tracer(tracer):
+    global _tracer
+    _tracer = tracer
+
+
+def _call(name, M, N, K, fn, *args):
+    if _tracer is None:
+        return _lib.check(fn(*args))
+    _tracer.begin(name, M, N, K)
+    try:
+        return _lib.check(fn(*args))
+    finally:
+        _tracer.end()
+
 
 def _stream():
     return torch.cuda.current_stream().cuda_stream
@@ -37,8 +56,8 @@ def dequant_interleaved_int4_to_fp16(output, qweight, scale, scaled_zero, group_
     _need(scale, torch.float16, "scale"); _need(scaled_zero, torch.float16, "scaled_zero")
     N, K = qweight.shape[0] * 4, qweight.shape[1]
     fn = _lib.load().kmi_cvt_i4_to_f16_tiled if tiled else _lib.load().kmi_cvt_i4_to_f16
-    _lib.check(fn(output.data_ptr(), qweight.data_ptr(), scale.data_ptr(), scaled_zero.data_ptr(),
-                  N, K, group_size, _stream()))
+    _call("cvt_i4_to_f16", 0, N, K, fn, output.data_ptr(), qweight.data_ptr(), scale.data_ptr(),
+          scaled_zero.data_ptr(), N, K, group_size, _stream())
 
 
 def dequant_interleaved_int4_to_int8(output, qweight, scale, scaled_zero, group_size=GROUP_SIZE, tiled=False):
@@ -47,8 +66,8 @@ def dequant_interleaved_int4_to_int8(output, qweight, scale, scaled_zero, group_
     _need(scale, torch.float16, "scale"); _need(scaled_zero, torch.float16, "scaled_zero")
     N, K = qweight.shape[0] * 4, qweight.shape[1]
     fn = _lib.load().kmi_cvt_i4_to_i8_tiled if tiled else _lib.load().kmi_cvt_i4_to_i8
-    _lib.check(fn(output.data_ptr(), qweight.data_ptr(), scale.data_ptr(), scaled_zero.data_ptr(),
-                  N, K, group_size, _stream()))
+    _call("cvt_i4_to_i8", 0, N, K, fn, output.data_ptr(), qweight.data_ptr(), scale.data_ptr(),
+          scaled_zero.data_ptr(), N, K, group_size, _stream())
 
 
 def untile(tiled, N, K):
@@ -64,7 +83,8 @@ def quant_fp16_to_int8(out, input, scale):
     _need(out, torch.int8, "out"); _need(input, torch.float16, "input"); _need(scale, torch.float16, "scale")
     K = input.shape[-1]
     M = input.numel() // K if K else 0
-    _lib.check(_lib.load().kmi_quant_act_i8(out.data_ptr(), scale.data_ptr(), input.data_ptr(), M, K, _stream()))
+    _call("quant_act_i8", M, 0, K, _lib.load().kmi_quant_act_i8, out.data_ptr(), scale.data_ptr(), input.data_ptr(),
+          M, K, _stream())
 
 
 # ---- products -----------------------------------------------------------------------------------
@@ -77,13 +97,9 @@ def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZ
     _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
     out = torch.empty(x.shape[:-1] + (n,), dtype=torch.float16, device=x.device)
     lib = _lib.load()
-    if cfg is None:
-        rc = lib.kmi_gemv_w4a16(out.data_ptr(), x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
-                                scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, _stream())
-    else:
-        rc = lib.kmi_gemv_w4a16_cfg(out.data_ptr(), x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
-                                    scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, cfg[0], cfg[1], _stream())
-    _lib.check(rc)
+    nt, nw = cfg if cfg is not None else (0, 0)
+    _call("gemv_w4a16", m, n, k, lib.kmi_gemv_w4a16_cfg, out.data_ptr(), x.data_ptr(), qweight.data_ptr(),
+          scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, _stream())
     return out
 
 
@@ -93,8 +109,9 @@ def gemm_forward(x, qweight, scales, scaled_zeros, bias=None):
     N, K = qweight.shape[0] * 4, qweight.shape[1]
     x2 = _flat2d(x)
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
-    _lib.check(_lib.load().kmi_gemm_w4a16(out.data_ptr(), x2.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
-                                          scaled_zeros.data_ptr(), _ptr(bias), x2.shape[0], N, K, GROUP_SIZE, _stream()))
+    _call("gemm_w4a16", x2.shape[0], N, K, _lib.load().kmi_gemm_w4a16, out.data_ptr(), x2.data_ptr(),
+          qweight.data_ptr(), scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), x2.shape[0], N, K,
+          GROUP_SIZE, _stream())
     return out
 
 
@@ -104,8 +121,8 @@ def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, 
     M, K = in_feats.shape
     N = out_feats.shape[-1]
     fn = _lib.load().kmi_gemm_w8a8_tiled if tiled else _lib.load().kmi_gemm_w8a8
-    _lib.check(fn(out_feats.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), wscales.data_ptr(),
-                  ascales.data_ptr(), _ptr(bias), M, N, K, _stream()))
+    _call("gemm_w8a8", M, N, K, fn, out_feats.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), wscales.data_ptr(),
+          ascales.data_ptr(), _ptr(bias), M, N, K, _stream())
 
 
 def w8a8_gemm_acc_i32(in_feats, kernel, N):
@@ -124,7 +141,8 @@ def w8a16_gemm_forward(x, w8, wscales, N, bias=None, tiled=False):
     M, K = x2.shape
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
     fn = _lib.load().kmi_gemm_w8a16_tiled if tiled else _lib.load().kmi_gemm_w8a16
-    _lib.check(fn(out.data_ptr(), x2.data_ptr(), w8.data_ptr(), wscales.data_ptr(), _ptr(bias), M, N, K, _stream()))
+    _call("gemm_w8a16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w8.data_ptr(), wscales.data_ptr(), _ptr(bias),
+          M, N, K, _stream())
     return out
 
 
@@ -135,8 +153,13 @@ def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
     M, K = x2.shape
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
     fn = _lib.load().kmi_gemm_f16_tiled if tiled else _lib.load().kmi_gemm_f16
-    _lib.check(fn(out.data_ptr(), x2.data_ptr(), w16.data_ptr(), _ptr(bias), M, N, K, _stream()))
+    _call("gemm_f16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w16.data_ptr(), _ptr(bias), M, N, K, _stream())
     return out
+
+
+def gemm_tile_for(M, N):
+    """Workgroup tile (64/128/256) the automatic choice uses for an M x N output."""
+    return _lib.load().kmi_gemm_pick_tile(int(M), int(N))
 
 
 def force_gemm_tile(tile):

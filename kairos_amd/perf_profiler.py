@@ -1,0 +1,160 @@
+"""Offline profiler and interval lookup table (kairos/perf_profiler.py:17-166).
+
+`Profiler(shape_list)` owns one LUT per (N, K) shape.  `profiling()` times every candidate lane of a
+DynamicLinear of that shape over a grid of M on the current GPU -- the timed call is `_forward`, so
+weight conversion, activation quantisation and output allocation are inside the measurement -- and
+run-length compresses the winners into segments.  `save`/`load` use the reference's file:
+`<dir>/seg_perf_list.pt`, JSON text, one list per shape of `[m_right_edge, lane_name, gain_pct]`.
+"""
+import json
+import os
+
+import torch
+
+from . import _lib
+from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+from .perf_eval import timer
+
+print_flag = False
+
+# M grid of the reference (perf_profiler.py:88-90)
+DEFAULT_INPUT_LEN = [1, 2, 4, 8, 16, 24, 32, 48, 64, 128, 256, 512] + \
+                    [i for i in range(1024, 1024 * 8, 1024)] + \
+                    [i for i in range(1024 * 8, 1024 * 32, 2048)]
+# candidate lanes: the reference's four plus W8A16, which exists on this hardware
+DEFAULT_COMP_TYPES = ['fp16', 'w4a16_gemm', 'w4a16_gemv', 'w8a8', 'w8a16_gemm']
+GEMV_MAX_M = 64
+
+
+class LUT:
+    """Interval table backed by the C ABI (kmi_lut_*); same get/record/shrink_to_fit as LUT_module.LUT."""
+
+    def __init__(self):
+        self._lib = _lib.load()
+        self._h = self._lib.kmi_lut_new()
+        if not self._h:
+            raise MemoryError("kmi_lut_new failed")
+
+    def get(self, m):
+        return _lib.check(self._lib.kmi_lut_get(self._h, int(m)))
+
+    def record(self, r, comp_type_id):
+        _lib.check(self._lib.kmi_lut_record(self._h, int(r), int(comp_type_id)))
+
+    def shrink_to_fit(self):
+        _lib.check(self._lib.kmi_lut_shrink_to_fit(self._h))
+
+    def __len__(self):
+        return self._lib.kmi_lut_size(self._h)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.kmi_lut_free(h)
+
+
+def save_json(save_path, obj):
+    os.makedirs(os.path.dirname(save_path) or ".", exist_ok=True)
+    with open(save_path, "w") as f:
+        f.write(json.dumps(obj))
+
+
+def load_json(load_path):
+    with open(load_path) as f:
+        return json.load(f)
+
+
+class Profiler:
+    comp_type_name = COMP_TYPE_NAME
+    linear_cls = DynamicLinear
+
+    @torch.no_grad()
+    def __init__(self, shape_list) -> None:
+        self.shape_list = [tuple(s) for s in shape_list]
+        self.seg_perf_list = []
+        self.lut = {shape: LUT() for shape in self.shape_list}
+
+    def record_best_comp(self, shape, r, comp_type):
+        self.lut[tuple(shape)].record(r, self.comp_type_name[comp_type])
+
+    def profiling(self, **kwargs):
+        for shape in self.shape_list:
+            seg = test_perf(str(shape), shape[1], shape[0], False, linear_cls=self.linear_cls,
+                            comp_type_name=self.comp_type_name, **kwargs)
+            for t in seg:
+                self.record_best_comp(shape, t[0], t[1])
+            self.seg_perf_list.append([list(t) for t in seg])
+
+    def get_comp_type(self, shape, m):
+        return self.lut[shape].get(m)
+
+    def save(self, path='./prof/'):
+        save_json(os.path.join(path, 'seg_perf_list.pt'), self.seg_perf_list)
+
+    def load(self, path='./prof/'):
+        self.seg_perf_list = load_json(os.path.join(path, 'seg_perf_list.pt'))
+        if len(self.seg_perf_list) != len(self.shape_list):
+            raise ValueError(f"{path}: table holds {len(self.seg_perf_list)} shapes, profiler has {len(self.shape_list)}")
+        for shape, seg in zip(self.shape_list, self.seg_perf_list):
+            for t in seg:
+                self.record_best_comp(shape, t[0], t[1])
+
+
+def compress_segments(perf_list):
+    """Run-length compression of (m, best, gain) tuples: keep the last tuple of every run of equal
+    `best` (perf_profiler.py:150-156), so each kept m is the inclusive right edge of its segment."""
+    seg = []
+    prev = perf_list[0]
+    for t in perf_list:
+        if t[1] != prev[1]:
+            seg.append(prev)
+        prev = t
+    seg.append(prev)
+    return seg
+
+
+def lane_allowed(comp_type, m):
+    if 'gemv' in comp_type and m > GEMV_MAX_M:
+        return False
+    return True
+
+
+@torch.no_grad()
+def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200, preheat_time=20,
+              linear_cls=DynamicLinear, comp_type_name=COMP_TYPE_NAME, details=None):
+    """Times every allowed lane for every M and returns the compressed segment list for one shape."""
+    torch.manual_seed(10)
+    lin = torch.nn.Linear(in_features=K, out_features=N, bias=bias, dtype=torch.float16).cuda()
+    dlinear = linear_cls.from_module(lin, 'cuda')
+    del lin
+    input_len = list(input_len or DEFAULT_INPUT_LEN)
+    comp_type_list = list(comp_type_list or DEFAULT_COMP_TYPES)
+    perf_list = []
+    for m in input_len:
+        x = torch.randn((1, m, K), dtype=torch.float16, device='cuda')
+        best_t, best_comp = float('inf'), ''
+        orig_t = float('inf')
+        for comp in comp_type_list:
+            if not lane_allowed(comp, m):
+                continue
+            cid = comp_type_name[comp]
+            for _ in range(preheat_time):
+                dlinear._forward(x, m, cid)
+            rec = []
+            with timer(comp, n=n, recordList=rec, print_flag=print_flag):
+                for _ in range(n):
+                    dlinear._forward(x, m, cid)
+            t = rec[-1]
+            if details is not None:
+                details.append({"shape": [N, K], "m": m, "comp": comp, "ms": t})
+            if t < best_t:
+                best_t, best_comp = t, comp
+            if 'w4' in comp and t < orig_t:
+                orig_t = t
+        gain = (orig_t - best_t) * 100 / orig_t if orig_t < float('inf') else 0.0
+        perf_list.append((m, best_comp, gain))
+    seg = compress_segments(perf_list)
+    print('-' * 7 + f'N:{N:5d}  K:{K:5d}' + '-' * 7)
+    for t in seg:
+        print(f'm: {t[0]:5d}   best: {t[1]:12s}  speed up: {t[2]:4.2f}%')
+    return seg

@@ -62,10 +62,25 @@ def awq_position(n, k, K):
 
 
 def pack_int_awq(q):
-    """uint4 [N, K] (any integer dtype, values 0..15) -> int16 [N/4, K]."""
+    """uint4 [N, K] (any integer dtype, values 0..15) -> int16 [N/4, K].
+
+    Vectorised form of awq_position(): K splits as (block64, half, nibble, word8); the nibble axis is
+    folded into the bits of the word.  tests/test_oracle_layout.py checks it against the index
+    formula, against both statements of the reference and by brute force.
+    """
     q = np.asarray(q)
     N, K = q.shape
     assert N % INTERLEAVE == 0 and K % KSTRIDE == 0
+    v = (q.astype(np.uint16) & 0xF).reshape(N // 4, 4, K // 64, 2, 4, 8)      # quad,row,blk,half,nib,word
+    v = v.transpose(0, 2, 1, 3, 5, 4)                                          # quad,blk,row,half,word,nib
+    w = v[..., 0] | (v[..., 1] << 4) | (v[..., 2] << 8) | (v[..., 3] << 12)
+    return np.ascontiguousarray(w).reshape(N // 4, K).view(np.int16)
+
+
+def pack_int_awq_by_index(q):
+    """Same result through awq_position() element by element (slow; the definition)."""
+    q = np.asarray(q)
+    N, K = q.shape
     nn, kk = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
     word, nib = awq_position(nn, kk, K)
     out = np.zeros(N // 4 * K, dtype=np.uint16)
@@ -77,9 +92,16 @@ def unpack_int_awq(packed):
     """int16 [N/4, K] -> uint8 [N, K] with values 0..15 (inverse of pack_int_awq)."""
     packed = np.ascontiguousarray(packed)
     N4, K = packed.shape
-    N = N4 * 4
+    w = packed.view(np.uint16).reshape(N4, K // 64, 4, 2, 8)                   # quad,blk,row,half,word
+    nib = np.stack([(w >> s) & 0xF for s in (0, 4, 8, 12)], axis=-1)           # ... ,nib
+    return np.ascontiguousarray(nib.transpose(0, 2, 1, 3, 5, 4)).reshape(N4 * 4, K).astype(np.uint8)
+
+
+def unpack_int_awq_by_index(packed):
+    packed = np.ascontiguousarray(packed)
+    N4, K = packed.shape
     flat = packed.view(np.uint16).ravel()
-    nn, kk = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
+    nn, kk = np.meshgrid(np.arange(N4 * 4), np.arange(K), indexing="ij")
     word, nib = awq_position(nn, kk, K)
     return ((flat[word] >> (4 * nib).astype(np.uint16)) & 0xF).astype(np.uint8)
 
@@ -185,20 +207,23 @@ def _fma_f16(q, s, z):
     return (q.astype(np.float64) * s.astype(np.float64) + z.astype(np.float64)).astype(np.float16)
 
 
-def _expand_groups(table, N, K, group_size):
-    """[Gp, N] table -> [N, K] by repeating each used group row group_size times."""
-    ng = K // group_size
-    return np.repeat(np.asarray(table)[:ng, :N].T, group_size, axis=1)
-
-
 def dequant_to_f16(qweight, scales, scaled_zeros, group_size=GROUP):
     """kernels/csrc/kairos_kernel/dequant_awq_format/dequant_i4_to_f16.cu:14-36,40-151.
 
     W16[n, k] = fma_f16(q[n, k], scales[k/G, n], scaled_zeros[k/G, n]) -> fp16 [N, K] row-major.
     """
-    q = unpack_int_awq(qweight)
-    N, K = q.shape
-    return _fma_f16(q, _expand_groups(scales, N, K, group_size), _expand_groups(scaled_zeros, N, K, group_size))
+    qweight = np.ascontiguousarray(qweight)
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    ng = K // group_size
+    out = np.empty((N, K), dtype=np.float16)
+    step = 2048                                                 # rows per slab: bounds the fp64 temporaries
+    for r0 in range(0, N, step):
+        r1 = min(N, r0 + step)
+        q = unpack_int_awq(qweight[r0 // 4:r1 // 4]).reshape(r1 - r0, ng, group_size)
+        s = np.asarray(scales)[:ng, r0:r1].T[:, :, None]
+        z = np.asarray(scaled_zeros)[:ng, r0:r1].T[:, :, None]
+        out[r0:r1] = _fma_f16(q, s, z).reshape(r1 - r0, K)
+    return out
 
 
 def dequant_to_i8(qweight, scales_to8, scaled_zeros_to8, group_size=GROUP):

@@ -1,0 +1,125 @@
+"""GPU tests of the module layer: DynamicLinear / SwitchLinear forward through every lane against
+the oracle's switched_forward, LUT-driven dispatch, temp-cache behaviour and the profiler loop."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from oracle import kairos_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda")
+
+
+def make_linear(N, K, bias, seed=10):
+    w = O.synth_weights(N, K, seed)
+    lin = torch.nn.Linear(K, N, bias=bias, dtype=torch.float16)
+    with torch.no_grad():
+        lin.weight.copy_(torch.from_numpy(w))
+        if bias:
+            lin.bias.copy_(torch.from_numpy(np.random.default_rng(seed).standard_normal(N).astype(np.float16)))
+    return lin, w
+
+
+@pytest.mark.parametrize("cls_name", ["DynamicLinear", "SwitchLinear"])
+@pytest.mark.parametrize("bias", [False, True])
+def test_every_lane_matches_oracle(gpu, cls_name, bias):
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos.switch_linear import SwitchLinear
+    cls = {"DynamicLinear": DynamicLinear, "SwitchLinear": SwitchLinear}[cls_name]
+    N, K = 256, 1024
+    lin, w = make_linear(N, K, bias)
+    dl = cls.from_module(lin.cuda(), 'cuda')
+    prep = O.prepare_weights(w)
+    for key in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1"):
+        got = getattr(dl, key).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), prep[key].view(np.uint16)), key   # GPU-side prep == oracle
+    b = lin.bias.detach().cpu().numpy() if bias else None
+    for M in (1, 9, 40, 200):
+        x = O.synth_acts(M, K, seed=M)
+        xd = torch.from_numpy(x).cuda()[None]
+        for name, cid in COMP_TYPE_NAME.items():
+            out = dl._forward(xd, M, cid)
+            assert out.shape == (1, M, N) and out.dtype == torch.float16
+            ref = O.switched_forward(x, prep, cid, bias=b)
+            err = O.max_abs_rel(out[0].cpu().numpy(), ref)
+            assert err < 1e-2, (name, M, err)
+            if name == "w8a8":
+                assert np.array_equal(out[0].cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_forward_uses_lut_and_counts_switches(gpu, tmp_path):
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos.perf_profiler import Profiler
+    N, K = 256, 512
+    prof = Profiler([(N, K)])
+    for r, name in [(4, 'w4a16_gemv'), (64, 'w4a16_gemm'), (512, 'w8a8'), (4096, 'fp16')]:
+        prof.record_best_comp((N, K), r, name)
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        lin, w = make_linear(N, K, False)
+        dl = DynamicLinear.from_module(lin.cuda(), 'cuda')
+        prep = O.prepare_weights(w)
+        seen = []
+        for B, S in [(1, 1), (1, 4), (2, 3), (2, 32), (4, 100), (3, 300), (1, 2)]:
+            x = O.synth_acts(B * S, K, seed=B * S)
+            out = dl(torch.from_numpy(x).cuda().reshape(B, S, K))
+            assert out.shape == (B, S, N)
+            m = B * S
+            want = prof.get_comp_type((N, K), m)
+            assert dl.comp_type == want and dl.pre_m == m
+            seen.append(want)
+            ref = O.switched_forward(x, prep, want)
+            assert O.max_abs_rel(out.reshape(m, N).cpu().numpy(), ref) < 1e-2
+        assert seen == [1, 1, 0, 0, 2, 5, 1]
+        assert dl.switch_count == 4
+    finally:
+        DynamicLinear.prof = old
+
+
+def test_temp_cache_reuse_and_bound(gpu):
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos_amd.temp_cache import TempCache
+    cache = TempCache()
+    a = DynamicLinear.from_module(make_linear(256, 512, False, 1)[0].cuda(), 'cuda')
+    b = DynamicLinear.from_module(make_linear(128, 1024, False, 2)[0].cuda(), 'cuda')
+    a.temp_cache = b.temp_cache = cache
+    x5 = torch.randn(1, 70, 512, dtype=torch.float16, device='cuda')
+    xb = torch.randn(1, 70, 1024, dtype=torch.float16, device='cuda')
+    o1 = a._forward(x5, 70, COMP_TYPE_NAME['w8a8'])
+    o2 = a._forward(x5, 70, COMP_TYPE_NAME['w8a8'])
+    assert cache.misses == 1 and cache.hits == 1 and torch.equal(o1, o2)
+    o3 = a._forward(x5, 70, COMP_TYPE_NAME['fp16'])              # other format: converts again
+    assert cache.misses == 2
+    b._forward(xb, 70, COMP_TYPE_NAME['fp16'])                   # other layer evicts
+    o4 = a._forward(x5, 70, COMP_TYPE_NAME['fp16'])
+    assert cache.misses == 4 and torch.equal(o3, o4)
+    assert cache.peak_bytes == 256 * 512 * 2 == max(256 * 512, 128 * 1024) * 2
+    assert cache.capacity == cache.peak_bytes                    # one buffer, sized by the largest request
+
+
+def test_profiler_builds_a_table(gpu, tmp_path):
+    from kairos.perf_profiler import Profiler
+    prof = Profiler([(256, 512)])
+    details = []
+    prof.profiling(input_len=[1, 16, 64, 128, 512], n=5, preheat_time=2, details=details)
+    seg = prof.seg_perf_list[0]
+    assert seg[-1][0] == 512 and all(t[1] in O.COMP_TYPE_NAME for t in seg)
+    assert not any(d["comp"] == "w4a16_gemv" and d["m"] > 64 for d in details)
+    assert {d["comp"] for d in details} == {'fp16', 'w4a16_gemm', 'w4a16_gemv', 'w8a8', 'w8a16_gemm'}
+    prof.save(str(tmp_path) + "/")
+    again = Profiler([(256, 512)])
+    again.load(str(tmp_path) + "/")
+    for m in (1, 16, 17, 100, 512, 5000):
+        assert again.get_comp_type((256, 512), m) == prof.get_comp_type((256, 512), m)
+    text = open(tmp_path / "seg_perf_list.pt").read()
+    assert json.loads(text) == prof.seg_perf_list

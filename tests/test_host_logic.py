@@ -1,0 +1,114 @@
+"""Host-side mirror of the reference interface, on CPU: table files, LUT wrapper, segment
+compression, module construction, the import-path aliases, and loud failure without a GPU."""
+import json
+import os
+import shutil
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kairos_oracle as O
+
+LLAMA_SHAPES = [(1024, 4096), (4096, 4096), (4096, 14336), (14336, 4096)]
+QWEN_SHAPES = [(512, 3584), (3584, 3584), (3584, 18944), (18944, 3584)]
+
+
+def test_alias_package_exposes_reference_names():
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos.dynamic_linear_v2 import COMP_TYPE_NAME as V2, DynamicLinear as D2
+    from kairos.switch_linear import SwitchLinear
+    from kairos.perf_profiler import LUT, Profiler, test_perf
+    from kairos.perf_profiler_v2 import Profiler as P2
+    from kairos.quantization import quantize_tensor_int8
+    import kairos_amd.dynamic_linear as impl
+    assert DynamicLinear is impl.DynamicLinear
+    assert COMP_TYPE_NAME == {'w4a16_gemm': 0, 'w4a16_gemv': 1, 'w8a8': 2, 'w8a16_gemm': 3, 'w8a16_gemv': 4, 'fp16': 5}
+    assert V2['w4a16_marlin'] == 6 and V2['w4a8_qserve'] == 7 and V2['fp16'] == 5
+    assert issubclass(SwitchLinear, D2) and P2.linear_cls is D2
+    assert callable(test_perf) and callable(quantize_tensor_int8) and LUT and Profiler
+
+
+@pytest.mark.parametrize("fixture,shapes", [("prof_llama_seg_perf_list.json", LLAMA_SHAPES),
+                                            ("prof_qwen_seg_perf_list.json", QWEN_SHAPES)])
+def test_profiler_loads_reference_tables(tmp_path, golden_dir, fixture, shapes):
+    from kairos.perf_profiler_v2 import Profiler
+    d = tmp_path / "prof"
+    d.mkdir()
+    shutil.copy(os.path.join(golden_dir, fixture), d / "seg_perf_list.pt")
+    prof = Profiler(shapes)
+    prof.load(str(d) + "/")
+    segs = json.load(open(os.path.join(golden_dir, fixture)))
+    for shape, seg in zip(shapes, segs):
+        want = O.LUT()
+        for r, name, _ in seg:
+            want.record(r, O.COMP_TYPE_NAME[name])
+        for m in [1, 2, 3, 7, 8, 9, 16, 17, 64, 65, 256, 257, 512, 1024, 1025, 4096, 22528, 22529, 30720, 99999]:
+            assert prof.get_comp_type(shape, m) == want.get(m)
+    # save writes the same JSON text format back
+    out = tmp_path / "out"
+    prof.save(str(out) + "/")
+    assert json.load(open(out / "seg_perf_list.pt")) == segs
+
+
+def test_v1_profiler_rejects_v2_only_lane(tmp_path, golden_dir):
+    from kairos.perf_profiler import Profiler
+    d = tmp_path / "prof"
+    d.mkdir()
+    shutil.copy(os.path.join(golden_dir, "prof_llama_seg_perf_list.json"), d / "seg_perf_list.pt")
+    with pytest.raises(KeyError):        # 'w4a16_marlin' is not in the v1 id table, as upstream
+        Profiler(LLAMA_SHAPES).load(str(d) + "/")
+
+
+def test_compress_segments_matches_reference_rule():
+    from kairos.perf_profiler import compress_segments
+    perf = [(1, 'w4a16_gemv', 0.0), (2, 'w4a16_gemv', 0.0), (4, 'w4a16_gemm', 0.0), (8, 'w4a16_gemm', 0.0),
+            (16, 'w8a8', 12.5), (32, 'w8a8', 30.0)]
+    assert compress_segments(perf) == [(2, 'w4a16_gemv', 0.0), (8, 'w4a16_gemm', 0.0), (32, 'w8a8', 30.0)]
+    assert compress_segments([(1, 'fp16', 1.0)]) == [(1, 'fp16', 1.0)]
+
+
+def test_lut_wrapper():
+    from kairos.perf_profiler import LUT
+    lut = LUT()
+    for r, c in [(8, 1), (256, 0), (30720, 2)]:
+        lut.record(r, c)
+    lut.shrink_to_fit()
+    assert len(lut) == 3
+    assert [lut.get(m) for m in (1, 8, 9, 256, 257, 10 ** 6, 9, 9)] == [1, 1, 0, 0, 2, 2, 0, 0]
+    from kairos_amd._lib import KairosMiError
+    with pytest.raises(KairosMiError):
+        LUT().get(5)
+
+
+def test_from_module_on_cpu_matches_oracle_and_refuses_cpu_compute():
+    from kairos.dynamic_linear import DynamicLinear
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(256, 64, bias=True, dtype=torch.float16)
+    dl = DynamicLinear.from_module(lin, 'cpu')
+    ref = O.prepare_weights(lin.weight.detach().numpy())
+    for key in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1"):
+        assert np.array_equal(getattr(dl, key).numpy().view(np.uint16), ref[key].view(np.uint16)), key
+    assert dl.shape == (64, 256) and dl.pre_m == 0 and dl.group_size == 128
+    assert torch.equal(dl.bias, lin.bias.detach())
+    assert "in_features=256, out_features=64, bias=True" in repr(dl)
+    empty = DynamicLinear.from_module(lin, 'cpu', init_only=True)
+    assert empty.qweight is None
+    with pytest.raises((ValueError, ImportError)):      # no CPU fallback: the HIP path is the only path
+        dl._forward(torch.zeros(1, 2, 256, dtype=torch.float16), 2, 1)
+
+
+def test_temp_cache_is_bounded_and_reuses():
+    from kairos_amd.temp_cache import TempCache
+    c = TempCache(capacity_limit=1024)
+    a, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert not hit and a.shape == (4, 64) and a.dtype == torch.int8
+    b, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert hit and b.data_ptr() == a.data_ptr()
+    d, hit = c.get(2, 'f16', (4, 64), torch.float16, 'cpu')
+    assert not hit and d.dtype == torch.float16 and c.capacity == 512 and c.peak_bytes == 512
+    _, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert not hit                                      # evicted by the other layer
+    with pytest.raises(MemoryError):
+        c.get(3, 'f16', (4, 256), torch.float16, 'cpu')
+    assert c.capacity <= 1024

@@ -48,6 +48,8 @@ def test_three_statements_agree(N, K):
     a = O.pack_int_awq(q)
     assert a.dtype == np.int16 and a.shape == (N // 4, K)
     assert np.array_equal(a, pack_stepwise(q))
+    assert np.array_equal(a, O.pack_int_awq_by_index(q))
+    assert np.array_equal(O.unpack_int_awq_by_index(a), q)
     assert np.array_equal(a, pack_closed_form(q))
     assert np.array_equal(O.unpack_int_awq(a), q)
     assert np.array_equal(unpack_closed_form(a), q)
