@@ -159,9 +159,7 @@ def main():
     # ---- synthetic layer copies --------------------------------------------------------------
     layers = []
     for _name, N, K in LAYER:
-        w = torch.from_numpy(O.synth_weights(N, K, seed=10)).to(dev)
-        prep = prepare_linear_weight(w)
-        del w
+        prep = {k: v.to(dev) for k, v in prepare_linear_weight(torch.from_numpy(O.synth_weights(N, K, seed=10))).items()}
         copies = []
         for c in range(args.copies):
             dl = DynamicLinear(K, N, False, dev, 128)

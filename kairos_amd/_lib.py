@@ -59,6 +59,10 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    # PyTorch ships its own HIP runtime under the same soname as the system one.  It must be the
+    # first (and only) copy in the process, so that streams, events and allocations are shared
+    # between torch and this library: load torch before dlopen-ing anything that needs the runtime.
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m kairos_amd.build` "

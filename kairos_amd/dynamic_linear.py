@@ -59,7 +59,10 @@ class DynamicLinear(torch.nn.Module):
         q_linear = cls(linear.in_features, linear.out_features, linear.bias is not None, device, group_size=128)
         if init_only:
             return q_linear
-        prepared = prepare_linear_weight(linear.weight.data, group_size=128)
+        # Quantisation runs on the host: ROCm PyTorch's elementwise fp32 division is not correctly
+        # rounded, so the same torch ops on the GPU flip round-half-even ties and give a (slightly)
+        # different int4 tensor than the reference arithmetic.  The packed result is then uploaded.
+        prepared = prepare_linear_weight(linear.weight.data.detach().cpu(), group_size=128)
         for key, value in prepared.items():
             setattr(q_linear, key, value.to(device))
         if linear.bias is not None:

@@ -158,3 +158,35 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
     for t in seg:
         print(f'm: {t[0]:5d}   best: {t[1]:12s}  speed up: {t[2]:4.2f}%')
     return seg
+
+
+PRESETS = {
+    # fused qkv / gate_up shapes of one decoder layer, (N, K)
+    "llama3_8b": [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)],
+    "llama3_8b_unfused": [(1024, 4096), (4096, 4096), (14336, 4096), (4096, 14336)],
+    "llama3_70b": [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)],
+    "qwen25_7b": [(4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)],
+}
+
+
+def main(argv=None):
+    import argparse
+    ap = argparse.ArgumentParser(description="Rebuild the per-shape M-interval table on this GPU")
+    ap.add_argument("--preset", default="llama3_8b", choices=sorted(PRESETS))
+    ap.add_argument("--out", required=True, help="directory that receives seg_perf_list.pt (and timings.json)")
+    ap.add_argument("--n", type=int, default=200)
+    ap.add_argument("--preheat", type=int, default=20)
+    ap.add_argument("--max-m", type=int, default=30720)
+    args = ap.parse_args(argv)
+    grid = sorted(set([m for m in DEFAULT_INPUT_LEN if m <= args.max_m] + [1 << i for i in range(13)]))
+    prof = Profiler(PRESETS[args.preset])
+    details = []
+    prof.profiling(input_len=grid, n=args.n, preheat_time=args.preheat, details=details)
+    out = args.out if args.out.endswith("/") else args.out + "/"
+    prof.save(out)
+    save_json(os.path.join(out, "timings.json"), details)
+    print(f"wrote {out}seg_perf_list.pt")
+
+
+if __name__ == "__main__":
+    main()
