@@ -76,6 +76,11 @@ class Tracer:
         ev.record()
         self.records.append(self._cur + (ev,))
 
+    def per_launch(self):
+        self.torch.cuda.synchronize()
+        return [{"label": l, "M": M, "N": N, "K": K, "us": round(e0.elapsed_time(e1) * 1e3, 2)}
+                for l, _n, M, N, K, e0, e1 in self.records]
+
     def summarise(self):
         self.torch.cuda.synchronize()
         agg = {}
@@ -180,7 +185,9 @@ def main():
         prof.load(LUT_DIR + "/")
     else:
         lut_source = "profiled at start-up (n=20)"
-        prof.profiling(input_len=M_GRID, n=20, preheat_time=5)
+        import contextlib
+        with contextlib.redirect_stdout(sys.stderr):
+            prof.profiling(input_len=M_GRID, n=20, preheat_time=5)
     DynamicLinear.prof = prof
 
     def step(s):
@@ -274,13 +281,6 @@ def main():
                                   "tflops": round(f / us / 1e6, 2), "gbps": round(b / us / 1e3, 1), "bound": bnd,
                                   "roofline_frac": round(ideal * 1e6 / us, 4),
                                   "lut_pick": names[prof.get_comp_type((N, K), M)] == lane})
-        out = args.out or os.path.join(ROOT, "gpurun_out", "bench_sweep.json")
-        try:
-            os.makedirs(os.path.dirname(out), exist_ok=True)
-            with open(out, "w") as fh:
-                json.dump({"sweep": sweep, "by_m_us_per_layer": by_m, "kernels": kernels}, fh, indent=1)
-        except OSError:
-            pass
         print(f"{'shape':8s} {'M':>5s} " + " ".join(f"{l:>18s}" for l in lanes), file=sys.stderr)
         for lname, N, K in LAYER:
             for M in M_GRID:
@@ -290,6 +290,15 @@ def main():
                     cells.append(f"{r[0]['us']:9.1f}us {100 * r[0]['roofline_frac']:5.1f}%{'*' if r[0]['lut_pick'] else ' '}"
                                  if r else " " * 18)
                 print(f"{lname:8s} {M:5d} " + " ".join(cells), file=sys.stderr)
+
+    out = args.out or os.path.join(ROOT, "gpurun_out", "bench_sweep.json")
+    try:
+        os.makedirs(os.path.dirname(out), exist_ok=True)
+        with open(out, "w") as fh:
+            json.dump({"sweep": sweep, "by_m_us_per_layer": by_m, "kernels": kernels,
+                       "launches": tracer.per_launch()}, fh, indent=1)
+    except OSError:
+        pass
 
     # best roofline fractions in the two regimes the targets name
     def best(pred):
