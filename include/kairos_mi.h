@@ -56,10 +56,11 @@ int kmi_cvt_i4_to_f16(void* out_f16, const void* qweight, const void* scales, co
 int kmi_cvt_i4_to_i8(void* out_i8, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
                      int N, int K, int G, void* stream);
 
-/* The same two conversions, written in the tiled layout the MFMA GEMMs stage straight into LDS:
- * [N/KMI_TILE_N][K/kb][KMI_TILE_N rows][128 bytes], kb = 64 (fp16) or 128 (int8), each row's eight
- * 16-byte chunks XOR-swizzled by ((row>>1)&7).  No reference counterpart exists (the reference's
- * permute_weight.cu is an uncompiled stub).  Needs N%KMI_TILE_N==0. */
+/* The same two conversions, written in the tiled layout the MFMA GEMMs copy straight into LDS:
+ * [N/KMI_TILE_N][K/kb][KMI_TILE_N rows][64 bytes], kb = 32 (fp16) or 64 (int8); inside a tile row r
+ * sits at r*64 and its four 16-byte chunks are XOR-swizzled: chunk c is stored at c ^ ((r>>2)&3).
+ * No reference counterpart exists (the reference's permute_weight.cu is an uncompiled stub).
+ * Needs N%KMI_TILE_N==0. */
 #define KMI_TILE_N 128
 int kmi_cvt_i4_to_f16_tiled(void* out_f16, const void* qweight, const void* scales, const void* scaled_zeros,
                             int N, int K, int G, void* stream);
@@ -119,8 +120,6 @@ int kmi_gemm_f16(void* out_f16, const void* x_f16, const void* w16, const void* 
 /* Variants reading the weight operand in the tiled layout written by kmi_cvt_*_tiled. */
 int kmi_gemm_w8a8_tiled(void* out_f16, const void* a8, const void* w8_tiled, const void* wscales_f16,
                         const void* ascales_f16, const void* bias, int M, int N, int K, void* stream);
-int kmi_gemm_w8a16_tiled(void* out_f16, const void* x_f16, const void* w8_tiled, const void* wscales_f16,
-                         const void* bias, int M, int N, int K, void* stream);
 int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, const void* bias,
                        int M, int N, int K, void* stream);
 

@@ -30,7 +30,6 @@ SIGNATURES = {
     "kmi_gemm_w8a8_acc_i32": [_P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_f16": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_w8a16_tiled": [_P, _P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_force_tile": [_I],
     "kmi_gemm_pick_tile": [_I, _I],

@@ -64,27 +64,27 @@ __global__ __launch_bounds__(256) void cvt_i4_kernel(void* __restrict__ out, con
         u4_t hi = {c[0], c[1], d[0], d[1]};
         o[0] = lo; o[1] = hi;
     } else if constexpr (OUT == OUT_F16_TILED) {
-        // tile = 128 rows x 64 fp16 (16 KiB); chunk c of row r sits at c ^ ((r>>1)&7)
+        // tile = 128 rows x 32 fp16 (8 KiB): this thread's 32 weights are exactly one tile row;
+        // chunk c of row r sits at c ^ ((r>>2)&3)
+        const int row = n & (KMI_TILE_N - 1);
+        const long tile = (long)(n / KMI_TILE_N) * (K >> 5) + (kb64 * 2 + h);
+        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 64) + row * 64;
+        const int sw = (row >> 2) & 3;
+        *reinterpret_cast<h8_t*>(base + ((0 ^ sw) << 4)) = w0;
+        *reinterpret_cast<h8_t*>(base + ((1 ^ sw) << 4)) = w1;
+        *reinterpret_cast<h8_t*>(base + ((2 ^ sw) << 4)) = w2;
+        *reinterpret_cast<h8_t*>(base + ((3 ^ sw) << 4)) = w3;
+    } else {
+        // tile = 128 rows x 64 int8 (8 KiB): this thread's 32 weights are half of one tile row
         const int row = n & (KMI_TILE_N - 1);
         const long tile = (long)(n / KMI_TILE_N) * (K >> 6) + kb64;
-        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 128) + row * 128;
-        const int sw = (row >> 1) & 7;
-        *reinterpret_cast<h8_t*>(base + (((4 * h + 0) ^ sw) << 4)) = w0;
-        *reinterpret_cast<h8_t*>(base + (((4 * h + 1) ^ sw) << 4)) = w1;
-        *reinterpret_cast<h8_t*>(base + (((4 * h + 2) ^ sw) << 4)) = w2;
-        *reinterpret_cast<h8_t*>(base + (((4 * h + 3) ^ sw) << 4)) = w3;
-    } else {
-        // tile = 128 rows x 128 int8 (16 KiB)
-        const int row = n & (KMI_TILE_N - 1);
-        const long tile = (long)(n / KMI_TILE_N) * (K >> 7) + (kb64 >> 1);
-        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 128) + row * 128;
-        const int sw = (row >> 1) & 7;
-        const int c0 = (kb64 & 1) * 4 + h * 2;
+        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 64) + row * 64;
+        const int sw = (row >> 2) & 3;
         const u2_t a = h8_to_i8x8(w0), b = h8_to_i8x8(w1), c = h8_to_i8x8(w2), d = h8_to_i8x8(w3);
         u4_t lo = {a[0], a[1], b[0], b[1]};
         u4_t hi = {c[0], c[1], d[0], d[1]};
-        *reinterpret_cast<u4_t*>(base + (((c0 + 0) ^ sw) << 4)) = lo;
-        *reinterpret_cast<u4_t*>(base + (((c0 + 1) ^ sw) << 4)) = hi;
+        *reinterpret_cast<u4_t*>(base + (((2 * h + 0) ^ sw) << 4)) = lo;
+        *reinterpret_cast<u4_t*>(base + (((2 * h + 1) ^ sw) << 4)) = hi;
     }
 }
 
@@ -96,10 +96,10 @@ __global__ __launch_bounds__(256) void untile_kernel(u4_t* __restrict__ out, con
     const int row_chunks = (K * es) >> 4;        // chunks per matrix row
     const int n = (int)(i / row_chunks);
     const int cg = (int)(i - (long)n * row_chunks);
-    const int kt = cg >> 3, c = cg & 7;
+    const int kt = cg >> 2, c = cg & 3;
     const int row = n & (KMI_TILE_N - 1);
-    const long tile = (long)(n / KMI_TILE_N) * (row_chunks >> 3) + kt;
-    out[i] = in[tile * (KMI_TILE_N * 8) + row * 8 + (c ^ ((row >> 1) & 7))];
+    const long tile = (long)(n / KMI_TILE_N) * (row_chunks >> 2) + kt;
+    out[i] = in[tile * (KMI_TILE_N * 4) + row * 4 + (c ^ ((row >> 2) & 3))];
 }
 
 static int cvt_common(const char* fn, int kind, void* out, const void* qweight, const void* scales,
@@ -143,8 +143,8 @@ extern "C" int kmi_cvt_i4_to_i8_tiled(void* out, const void* qw, const void* s, 
 extern "C" int kmi_untile(void* out, const void* tiled, int N, int K, int elem_size, void* stream) {
     if (!out || !tiled) return kmi_set_error(KMI_E_NULL, "kmi_untile: NULL pointer argument");
     if (!kmi_aligned16(out) || !kmi_aligned16(tiled)) return kmi_set_error(KMI_E_ALIGN, "kmi_untile: pointers must be 16-byte aligned");
-    if ((elem_size != 1 && elem_size != 2) || N <= 0 || K <= 0 || (N % KMI_TILE_N) || ((K * elem_size) & 127))
-        return kmi_set_error(KMI_E_SHAPE, "kmi_untile: need elem_size in {1,2}, N%%%d==0, row bytes %%128==0 (N=%d K=%d es=%d)",
+    if ((elem_size != 1 && elem_size != 2) || N <= 0 || K <= 0 || (N % KMI_TILE_N) || ((K * elem_size) & 63))
+        return kmi_set_error(KMI_E_SHAPE, "kmi_untile: need elem_size in {1,2}, N%%%d==0, row bytes %%64==0 (N=%d K=%d es=%d)",
                              KMI_TILE_N, N, K, elem_size);
     const long chunks = (long)N * K * elem_size / 16;
     hipLaunchKernelGGL(untile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),

@@ -38,6 +38,150 @@ __device__ __forceinline__ void i8x4_to_h2x2(uint32_t w, h2_t& lo, h2_t& hi) {
     hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - k1152;
 }
 
+// Epilogue shared by both kernels.  The MFMAs are issued with the weight fragment as the first
+// operand, so an accumulator tile is D^T: lane (c = lane&31, hl = lane>>5) holds, for activation row
+// m = c, the output columns n = 8g + 4hl + r (e = 4g + r) -- four consecutive columns per g.
+// A wave converts one 32-row block at a time, writes it to its private LDS patch as fp16 [32][BN/2]
+// (8-byte writes, pitch padded by 8 bytes -> conflict free), and streams it out with 16-byte stores
+// in which 16 consecutive lanes cover 256 contiguous bytes of one output row.
+template <int KIND, int BM, int BN, bool HAS_BIAS, int FM, int FN, typename acc_t>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM][FN], char* smem, int m0, int n0,
+                                              int wave, int lane) {
+    const int M = p.M, N = p.N;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int c = lane & 31, hl = lane >> 5;
+#ifdef KMI_DBG_NOEPI
+    {   // keep the accumulators alive, store almost nothing
+        int sacc = 0;
+        for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int e = 0; e < 16; ++e) sacc += (int)acc[i][j][e];
+        if (sacc == 0x12345678) static_cast<int*>(p.out)[0] = sacc;
+        return;
+    }
+#endif
+    const int mw = m0 + wm * (BM / 2), nw = n0 + wn * (BN / 2);
+    if constexpr (KIND == KIND_W8A8_ACC) {
+        // raw accumulators (verification tier): plain element stores
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int m = mw + i * 32 + c;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int n = nw + j * 32 + 8 * (e >> 2) + 4 * hl + (e & 3);
+                    if (m < M && n < N) static_cast<int*>(p.out)[(long)m * N + n] = acc[i][j][e];
+                }
+        }
+    } else {
+        constexpr int WN = BN / 2;                       // columns per wave
+        constexpr int PITCH = WN * 2 + 8;                // bytes
+        constexpr int CPR = WN * 2 / 16;                 // 16-byte chunks per row
+        char* patch = smem + wave * (32 * PITCH);
+        // per-column factors of this lane: columns nw + j*32 + 8g + 4hl + (0..3), one 8-byte load each
+        // (N % 4 == 0, so a group of four columns is entirely inside or outside the matrix)
+        h4_t ws4[FN][4], bs4[FN][4];
+        (void)ws4; (void)bs4;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int n = nw + j * 32 + 8 * g + 4 * hl;
+                n = n < N ? n : N - 4;
+                if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) ws4[j][g] = *reinterpret_cast<const h4_t*>(p.wscales + n);
+                if constexpr (HAS_BIAS) bs4[j][g] = *reinterpret_cast<const h4_t*>(p.bias + n);
+            }
+        float as_i[FM];
+        (void)as_i;
+        if constexpr (KIND == KIND_W8A8) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                const int m = mw + i * 32 + c;
+                as_i[i] = (float)p.ascales[m < M ? m : M - 1];
+            }
+        }
+        half_t* outp = static_cast<half_t*>(p.out);
+        const bool wide = (N & 7) == 0;                  // 16-byte row segments stay aligned
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    half_t h[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float v;
+                        if constexpr (KIND == KIND_W8A8) {
+                            // product rounded to fp32 first, then to fp16 (two roundings, as the
+                            // reference epilogue): keep the compiler from fusing them into one
+                            v = (float)acc[i][j][4 * g + r] * ((float)ws4[j][g][r] * as_i[i]);
+                            asm volatile("" : "+v"(v));
+                        } else if constexpr (KIND == KIND_W8A16) {
+                            v = acc[i][j][4 * g + r] * (float)ws4[j][g][r];
+                        } else {
+                            v = acc[i][j][4 * g + r];
+                        }
+                        h[r] = (half_t)v;
+                        if constexpr (HAS_BIAS) h[r] = (half_t)((float)h[r] + (float)bs4[j][g][r]);
+                    }
+                    h4_t pk = {h[0], h[1], h[2], h[3]};
+                    *reinterpret_cast<h4_t*>(patch + c * PITCH + (j * 32 + 8 * g + 4 * hl) * 2) = pk;
+                }
+            // the patch is private to the wave and LDS serves a wave's requests in order
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int k = 0; k < 32 * CPR / 64; ++k) {
+                const int idx = k * 64 + lane, row = idx / CPR, ch = idx % CPR;
+                const u4_t v = *reinterpret_cast<const u4_t*>(patch + row * PITCH + ch * 16);
+                const int m = mw + i * 32 + row, n = nw + ch * 8;
+                if (m < M) {
+                    half_t* dst = outp + (long)m * N + n;
+                    if (wide) {
+                        if (n < N) *reinterpret_cast<u4_t*>(dst) = v;
+                    } else {                             // N % 8 == 4: two 8-byte halves, each whole or absent
+                        if (n < N) *reinterpret_cast<u2_t*>(dst) = u2_t{v[0], v[1]};
+                        if (n + 4 < N) *reinterpret_cast<u2_t*>(dst + 4) = u2_t{v[2], v[3]};
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
+        }
+    }
+}
+
+// Scheduling hints: spread READS LDS reads, WRITES LDS writes and LOADS global loads evenly between
+// the NMFMA MFMAs of one k-step, so that the matrix pipe never waits behind a burst of memory issue.
+template <int NMFMA, int READS, int WRITES, int LOADS, int K = 0>
+__device__ __forceinline__ void sched_interleave() {
+    if constexpr (NMFMA >= 4 && K < NMFMA) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int r = (K + 1) * READS / NMFMA - K * READS / NMFMA;
+        constexpr int w = (K + 1) * WRITES / NMFMA - K * WRITES / NMFMA;
+        constexpr int l = (K + 1) * LOADS / NMFMA - K * LOADS / NMFMA;
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+        if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
+        if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        sched_interleave<NMFMA, READS, WRITES, LOADS, K + 1>();
+    }
+}
+
+// Workgroup -> output tile.  Hardware deals workgroups round-robin over the 8 XCDs (id % 8), each
+// with a private L2.  Give every XCD a contiguous run of the tile sequence, and order that sequence
+// in column-major groups of GROUP_M tile rows, so the tiles resident on one XCD at a time form a
+// compact block that shares A row-panels and B column-panels in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int wg, int TM, int TN, int& tm, int& tn) {
+    constexpr int XCDS = 8, GROUP_M = 8;
+    const int total = TM * TN;
+    const int xcd = wg % XCDS, q = wg / XCDS;
+    const int base = total / XCDS, rem = total % XCDS;
+    const int L = xcd * base + (xcd < rem ? xcd : rem) + q;
+    const int per_group = GROUP_M * TN;
+    const int g = L / per_group, in_g = L - g * per_group;
+    const int rows = (TM - g * GROUP_M) < GROUP_M ? (TM - g * GROUP_M) : GROUP_M;
+    tn = in_g / rows;
+    tm = g * GROUP_M + (in_g - tn * rows);
+}
+
 template <int KIND, int BM, int BN, bool TILED_B>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     constexpr bool I8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
@@ -53,12 +197,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int M = p.M, N = p.N, K = p.K;
+    int tm, tn;
+    tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
     const long a_row_bytes = I8 ? (long)K : (long)K * 2;
     const int KT = (int)(a_row_bytes >> 7);
-    const char* A = static_cast<const char*>(p.a);
-    const char* B = static_cast<const char*>(p.b);
 
     acc_t acc[FM][FN];
 #pragma unroll
@@ -68,6 +212,45 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
+    // ---- per-thread global sources (rows beyond M / N are clamped: their products are never stored)
+    const char* pa[A_CH];
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+        const int q = tid + i * 256, row = q >> 3, c = q & 7;
+        int m = m0 + row;
+        m = m < M ? m : M - 1;
+        pa[i] = static_cast<const char*>(p.a) + (long)m * a_row_bytes + c * 16;
+    }
+    const char* pb[B_CH];
+    long b_step;                                              // bytes between consecutive k-tiles
+    int scale_col[B_CH];
+    (void)scale_col;
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+        const int q = tid + i * 256;
+        const char* B = static_cast<const char*>(p.b);
+        if constexpr (KIND == KIND_W4A16) {
+            const int row = q >> 1, h = q & 1;
+            int n = n0 + row;
+            n = n < N ? n : N - 1;
+            pb[i] = B + (long)(n >> 2) * K * 2 + (n & 3) * 32 + h * 16;
+            scale_col[i] = n;
+        } else if constexpr (KIND == KIND_W8A16) {
+            const int row = q >> 2, c = q & 3;
+            int n = n0 + row;
+            n = n < N ? n : N - 1;
+            pb[i] = B + (long)n * K + c * 16;
+        } else {
+            const int row = q >> 3, c = q & 7;
+            int n = n0 + row;
+            n = n < N ? n : N - 1;
+            pb[i] = B + (long)n * a_row_bytes + c * 16;
+        }
+    }
+    static_assert(!TILED_B, "the register-staged kernel reads row-major / packed operands only");
+    if constexpr (KIND == KIND_W8A16) b_step = 64;
+    else b_step = 128;
+
     u4_t ra[A_CH];
     u4_t rb[B_CH];
     half_t rs[B_CH], rz[B_CH];
@@ -75,64 +258,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
     auto load_tile = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < A_CH; ++i) {
-            const int q = tid + i * 256, row = q >> 3, c = q & 7;
-            const int m = m0 + row;
-            ra[i] = (m < M) ? *reinterpret_cast<const u4_t*>(A + (long)m * a_row_bytes + (long)kt * 128 + c * 16)
-                            : u4_t{0, 0, 0, 0};
-        }
-        if constexpr (KIND == KIND_W4A16) {
+        for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u4_t*>(pa[i] + (long)kt * 128);
 #pragma unroll
-            for (int i = 0; i < B_CH; ++i) {
-                const int q = tid + i * 256, row = q >> 1, h = q & 1;
-                int n = n0 + row;
-                n = n < N ? n : N - 1;
-                rb[i] = *reinterpret_cast<const u4_t*>(B + (long)(n >> 2) * K * 2 + (long)kt * 128 + (n & 3) * 32 + h * 16);
-                rs[i] = p.scales[(long)(kt >> 1) * N + n];
-                rz[i] = p.szeros[(long)(kt >> 1) * N + n];
-            }
-        } else if constexpr (TILED_B && KIND == KIND_W8A16) {
-            // int8 tiles are 128 K wide: this 64-wide k-tile is one half of every row of tile kt/2
-#pragma unroll
-            for (int i = 0; i < B_CH; ++i) {
-                const int q = tid + i * 256, row = q >> 2, c4 = q & 3;
-                const int strip = row >> 7, rin = row & 127;
-                if (n0 + strip * KMI_TILE_N < N) {
-                    const long tile = ((long)(n0 / KMI_TILE_N) + strip) * (K >> 7) + (kt >> 1);
-                    const int src_c = ((kt & 1) * 4 + c4) ^ ((rin >> 1) & 7);
-                    rb[i] = *reinterpret_cast<const u4_t*>(B + tile * (KMI_TILE_N * 128) + rin * 128 + src_c * 16);
-                } else {
-                    rb[i] = u4_t{0, 0, 0, 0};
-                }
-            }
-        } else if constexpr (TILED_B) {
-            // the k-tile of a 128-row strip is one contiguous, already swizzled 16 KiB block
-#pragma unroll
-            for (int i = 0; i < B_CH; ++i) {
-                const int q = tid + i * 256;                 // chunk index inside the BN x 128B tile
-                const int strip = q >> 10, inner = q & 1023;
-                if (n0 + strip * KMI_TILE_N < N) {
-                    const long tile = ((long)(n0 / KMI_TILE_N) + strip) * KT + kt;
-                    rb[i] = *reinterpret_cast<const u4_t*>(B + tile * (KMI_TILE_N * 128) + inner * 16);
-                } else {
-                    rb[i] = u4_t{0, 0, 0, 0};
-                }
-            }
-        } else if constexpr (KIND == KIND_W8A16) {
-#pragma unroll
-            for (int i = 0; i < B_CH; ++i) {
-                const int q = tid + i * 256, row = q >> 2, c = q & 3;
-                int n = n0 + row;
-                n = n < N ? n : N - 1;
-                rb[i] = *reinterpret_cast<const u4_t*>(B + (long)n * K + (long)kt * 64 + c * 16);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < B_CH; ++i) {
-                const int q = tid + i * 256, row = q >> 3, c = q & 7;
-                int n = n0 + row;
-                n = n < N ? n : N - 1;
-                rb[i] = *reinterpret_cast<const u4_t*>(B + (long)n * a_row_bytes + (long)kt * 128 + c * 16);
+        for (int i = 0; i < B_CH; ++i) {
+            rb[i] = *reinterpret_cast<const u4_t*>(pb[i] + (long)kt * b_step);
+            if constexpr (KIND == KIND_W4A16) {
+                rs[i] = p.scales[(long)(kt >> 1) * N + scale_col[i]];
+                rz[i] = p.szeros[(long)(kt >> 1) * N + scale_col[i]];
             }
         }
     };
@@ -171,9 +303,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
                 *reinterpret_cast<h8_t*>(sb + lds_off(row, 2 * c)) = lo;
                 *reinterpret_cast<h8_t*>(sb + lds_off(row, 2 * c + 1)) = hi;
             }
-        } else if constexpr (TILED_B) {
-#pragma unroll
-            for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u4_t*>(sb + (tid + i * 256) * 16) = rb[i];
         } else {
 #pragma unroll
             for (int i = 0; i < B_CH; ++i) {
@@ -183,83 +312,264 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
         }
     };
 
-    auto compute = [&](int stage) {
+    // ---- fragments: two register sets, read one k-step ahead of the MFMAs that consume them
+    u4_t fa[2][FM], fb[2][FN];
+    const int fr = lane & 31, fkh = lane >> 5;
+    auto read_frags = [&](int stage, int s, int set) {
         const char* sa = smem + stage * STAGE + (wm * (BM / 2)) * 128;
         const char* sb = smem + stage * STAGE + BM * 128 + (wn * (BN / 2)) * 128;
-        const int r = lane & 31, kh = lane >> 5;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            u4_t fa[FM], fb[FN];
+        for (int i = 0; i < FM; ++i) fa[set][i] = *reinterpret_cast<const u4_t*>(sa + lds_off(i * 32 + fr, 2 * s + fkh));
 #pragma unroll
-            for (int i = 0; i < FM; ++i) fa[i] = *reinterpret_cast<const u4_t*>(sa + lds_off(i * 32 + r, 2 * s + kh));
+        for (int j = 0; j < FN; ++j) fb[set][j] = *reinterpret_cast<const u4_t*>(sb + lds_off(j * 32 + fr, 2 * s + fkh));
+    };
+    auto mfma_step = [&](int set) {
 #pragma unroll
-            for (int j = 0; j < FN; ++j) fb[j] = *reinterpret_cast<const u4_t*>(sb + lds_off(j * 32 + r, 2 * s + kh));
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (I8)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i4_t, fb[set][j]),
+                                                                      __builtin_bit_cast(i4_t, fa[set][i]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, fb[set][j]),
+                                                                       __builtin_bit_cast(h8_t, fa[set][i]), acc[i][j], 0, 0, 0);
+            }
+    };
+    constexpr bool PURE_COPY = (KIND == KIND_F16 || I8);     // staging without conversion ALU work
+    constexpr int NMF = FM * FN, NRD = FM + FN, NWR = PURE_COPY ? A_CH + B_CH : 0, NLD = A_CH + B_CH;
+
+    // ---- software pipeline.  LDS stage t&1 holds k-tile t.  Per k-tile:
+    //   steps 0,1: MFMAs + fragment reads of the next step
+    //   step 2   : MFMAs + fragment reads of step 3 + write k-tile t+1 (already in registers) to the other stage
+    //   barrier  : the other stage is complete, this stage is no longer read
+    //   step 3   : MFMAs + fragment reads of step 0 of k-tile t+1 + global loads of k-tile t+2
+    load_tile(0);
+    store_tile(0);
+    if (KT > 1) load_tile(1);
+    __syncthreads();
+    read_frags(0, 0, 0);
+    for (int kt = 0; kt < KT - 1; ++kt) {
+        const int cur = kt & 1, nxt = cur ^ 1;
+        read_frags(cur, 1, 1);
+        mfma_step(0);
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(cur, 2, 0);
+        mfma_step(1);
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(cur, 3, 1);
+        store_tile(nxt);
+        mfma_step(0);
+        sched_interleave<NMF, NRD, NWR, 0>();
+        __syncthreads();
+        read_frags(nxt, 0, 0);
+        if (kt + 2 < KT) load_tile(kt + 2);
+        mfma_step(1);
+        sched_interleave<NMF, NRD, 0, NLD>();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    {   // last k-tile: nothing left to stage
+        const int cur = (KT - 1) & 1;
+        read_frags(cur, 1, 1);
+        mfma_step(0);
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(cur, 2, 0);
+        mfma_step(1);
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(cur, 3, 1);
+        mfma_step(0);
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step(1);
+    }
+
+    __syncthreads();                                         // staging LDS is reused by the epilogue
+    if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+    else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+}
+
+// =================================================================================================
+// Direct-to-LDS variant for the operand-copy kinds (KIND_F16, KIND_W8A8, KIND_W8A8_ACC).
+//
+// A lone workgroup of the register-staged kernel above spends ~1.9 us per 128-byte k-tile, against
+// 0.85 us of MFMA work: with one workgroup per CU the only way to cover the ~1.6 us global-load
+// latency is to keep several k-tiles in flight, and registers cannot hold them.  Here global loads
+// write LDS directly (global_load_lds_dwordx4: the 64 lanes of a wave fill one contiguous KiB), so
+// the spare LDS stages ARE the in-flight buffer: NS stages of (BM+BN) rows x 64 bytes, loads issued
+// NS-1 stages ahead, one barrier per stage.
+//
+// Stage layout: row r (A rows first, then B rows) at r*64; its four 16-byte chunks are stored at
+// c ^ ((r>>2)&3), which spreads the fragment reads of 16 consecutive rows over all 64 banks.  Since a
+// direct load puts lane l's data at slot l, the swizzle is applied on the global side: lane l
+// fetches the chunk that belongs in slot l.  The tiled weight layout ([N/128][K-stages][128][64 B],
+// already swizzled) makes the B side a straight 8 KiB copy per 128-row strip.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
+
+template <int KIND, int BM, int BN, bool TILED_B, int NS>
+__global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
+    constexpr bool I8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
+    static_assert(KIND == KIND_F16 || I8, "direct staging copies operands verbatim");
+    constexpr int FM = BM / 64, FN = BN / 64;
+    constexpr int ROWS = BM + BN;
+    constexpr int STAGE = ROWS * 64;
+    constexpr int NLD = ROWS * 4 / 256;                     // direct loads per thread per stage
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && NLD * 64 == ROWS, "each wave-load fills 16 rows");
+    using acc_t = typename std::conditional<I8, i16_t, f16_t>::type;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int M = p.M, N = p.N, K = p.K;
+    int tm, tn;
+    tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const long row_bytes = I8 ? (long)K : (long)K * 2;
+    const int T = (int)(row_bytes >> 6);                    // 64-byte stages along K
+
+    acc_t acc[FM][FN];
 #pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    if constexpr (I8)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i4_t, fa[i]),
-                                                                          __builtin_bit_cast(i4_t, fb[j]), acc[i][j], 0, 0, 0);
-                    else
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, fa[i]),
-                                                                           __builtin_bit_cast(h8_t, fb[j]), acc[i][j], 0, 0, 0);
-                }
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    // ---- global sources.  Load i of wave w fills the KiB region R = 4*i + w = rows 16R .. 16R+15.
+    const char* src[NLD];
+    long step[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int row = 16 * (4 * i + wave) + (lane >> 2);
+        const int pc = lane & 3;
+        const int c = pc ^ ((row >> 2) & 3);
+        if (16 * (4 * i) < BM) {                             // region lies in the A part (BM % 64 == 0)
+            int m = m0 + row;
+            m = m < M ? m : M - 1;
+            src[i] = static_cast<const char*>(p.a) + (long)m * row_bytes + c * 16;
+            step[i] = 64;
+        } else if constexpr (TILED_B) {
+            const int rb = row - BM;
+            int strip = rb >> 7;
+            if (n0 + strip * KMI_TILE_N >= N) strip = 0;
+            src[i] = static_cast<const char*>(p.b) + ((long)(n0 / KMI_TILE_N) + strip) * T * (KMI_TILE_N * 64) +
+                     (rb & 127) * 64 + pc * 16;
+            step[i] = KMI_TILE_N * 64;
+        } else {
+            int n = n0 + row - BM;
+            n = n < N ? n : N - 1;
+            src[i] = static_cast<const char*>(p.b) + (long)n * row_bytes + c * 16;
+            step[i] = 64;
+        }
+    }
+    auto issue_stage = [&](int t) {                          // k-stage t -> LDS stage t % NS
+        const int tt = t < T ? t : T - 1;                    // past the end: harmless reload into a free stage
+        char* dst = smem + (t % NS) * STAGE + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+#ifdef KMI_DBG_NOLOAD
+            if (t >= NS) continue;
+#endif
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(src[i] + tt * step[i]), (lds_void_ptr)(dst + i * 4096), 16, 0, 0);
         }
     };
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = (kt + 1 < KT);
-        if (more) load_tile(kt + 1);
-        compute(kt & 1);
-        if (more) store_tile((kt + 1) & 1);
-        __syncthreads();
+    // ---- fragment addressing: lane (r = lane&31, kh = lane>>5) reads chunk 2s+kh of row base+r
+    const int fr = lane & 31, fkh = lane >> 5;
+    const int fsw = (fr >> 2) & 3;
+    int off_a[2], off_b[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        off_a[s] = (wm * (BM / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
+        off_b[s] = (BM + wn * (BN / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
     }
-
-    // ---- epilogue: lane holds, per 32x32 tile, column (lane&31) and rows 8*(e/4) + 4*(lane>>5) + e%4
-    const int col_in = lane & 31, row_in = (lane >> 5) * 4;
+    u4_t fa[2][FM], fb[2][FN];
+    auto read_frags = [&](int t, int s, int set) {
+#ifdef KMI_DBG_NOREAD
+        if (t > 0) return;
+#endif
+        const char* st = smem + (t % NS) * STAGE;
 #pragma unroll
-    for (int j = 0; j < FN; ++j) {
-        const int n = n0 + wn * (BN / 2) + j * 32 + col_in;
-        if (n >= N) continue;
-        float ws = 1.0f, bv = 0.0f;
-        if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) ws = (float)p.wscales[n];
-        if (p.bias) bv = (float)p.bias[n];
+        for (int i = 0; i < FM; ++i) fa[set][i] = *reinterpret_cast<const u4_t*>(st + off_a[s] + i * 2048);
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
+        for (int j = 0; j < FN; ++j) fb[set][j] = *reinterpret_cast<const u4_t*>(st + off_b[s] + j * 2048);
+    };
+    auto mfma_step = [&](int set) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (e >> 2) + row_in + (e & 3);
-                if (m >= M) continue;
-                if constexpr (KIND == KIND_W8A8_ACC) {
-                    static_cast<int*>(p.out)[(long)m * N + n] = acc[i][j][e];
-                } else {
-                    float v;
-                    if constexpr (KIND == KIND_W8A8) {
-                        // product rounded to fp32 first, then to fp16 (two roundings, as the
-                        // reference epilogue): keep the compiler from fusing them into one
-                        v = (float)acc[i][j][e] * (ws * (float)p.ascales[m]);
-                        asm volatile("" : "+v"(v));
-                    }
-                    else if constexpr (KIND == KIND_W8A16) v = acc[i][j][e] * ws;
-                    else v = acc[i][j][e];
-                    half_t h = (half_t)v;
-                    if (p.bias) h = (half_t)((float)h + bv);
-                    static_cast<half_t*>(p.out)[(long)m * N + n] = h;
-                }
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (I8)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i4_t, fb[set][j]),
+                                                                      __builtin_bit_cast(i4_t, fa[set][i]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, fb[set][j]),
+                                                                       __builtin_bit_cast(h8_t, fa[set][i]), acc[i][j], 0, 0, 0);
             }
-        }
+    };
+    constexpr int NMF = FM * FN, NRD = FM + FN;
+
+    // Wait until at most `keep` direct loads of this thread are outstanding, then meet the other waves.
+    // A plain barrier instruction (no fence): the fence of __syncthreads would drain every load.
+#define KMI_STAGE_BARRIER(keep) asm volatile("s_waitcnt vmcnt(" #keep ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+    // ---- pipeline: stage t is computed while stages t+1 .. t+NS-1 are in flight.  The MFMAs run one
+    // k-step behind the fragment reads, across the barrier, so LDS latency is never exposed.
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t) issue_stage(t);
+    static_assert(NS == 4 || NS == 3, "vmcnt immediates below assume 3 or 4 stages");
+    if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);
+    else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);
+    else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);
+    else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);
+    else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);
+    else KMI_STAGE_BARRIER(0);
+    issue_stage(NS - 1);
+    read_frags(0, 0, 0);
+    read_frags(0, 1, 1);
+    for (int t = 0; t < T - 1; ++t) {
+        mfma_step(0);                                        // (t, step 0)
+        sched_interleave<NMF, 0, 0, 0>();
+        if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);
+        else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);
+        else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);
+        else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);
+        else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);
+        else KMI_STAGE_BARRIER(0);
+        // stage t+1 has landed for every wave; stage t is no longer read by anyone (its fragments
+        // for step 1 sit in registers), so it can take k-stage t+NS
+        issue_stage(t + NS);
+        read_frags(t + 1, 0, 0);
+        mfma_step(1);                                        // (t, step 1)
+        sched_interleave<NMF, NRD, 0, NLD>();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(t + 1, 1, 1);
     }
+    mfma_step(0);
+    mfma_step(1);
+    // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#undef KMI_STAGE_BARRIER
+
+    if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+    else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
 template <int KIND, int BM, int BN, bool TILED>
 static int launch_gemm(const GemmArgs& a, hipStream_t st) {
-    constexpr size_t lds = 2 * (size_t)(BM + BN) * 128;
-    auto fn = gemm_kernel<KIND, BM, BN, TILED>;
+    constexpr bool DIRECT = (KIND == KIND_F16 || KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
+    constexpr int NS = 4;
+    constexpr size_t lds = DIRECT ? (size_t)NS * (BM + BN) * 64 : 2 * (size_t)(BM + BN) * 128;
+    void (*fn)(GemmArgs);
+    if constexpr (DIRECT) fn = gemm_direct_kernel<KIND, BM, BN, TILED, NS>;
+    else fn = gemm_kernel<KIND, BM, BN, false>;
     if (lds > 64 * 1024) {
         static thread_local bool raised = false;   // per kernel instantiation, per thread
         if (!raised) {
@@ -268,7 +578,7 @@ static int launch_gemm(const GemmArgs& a, hipStream_t st) {
             raised = true;
         }
     }
-    const dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM), block(256);
+    const dim3 grid(((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM)), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     return KMI_OK;
 }
@@ -350,13 +660,6 @@ extern "C" int kmi_gemm_w8a8_tiled(void* out, const void* a8, const void* w8t, c
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8_tiled: NULL scale vector");
     GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K};
     KMI_GEMM_BODY("kmi_gemm_w8a8_tiled", KIND_W8A8, true)
-}
-
-extern "C" int kmi_gemm_w8a16_tiled(void* out, const void* x, const void* w8t, const void* wscales, const void* bias,
-                                    int M, int N, int K, void* stream) {
-    if (!wscales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a16_tiled: NULL wscales");
-    GemmArgs a{out, x, w8t, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K};
-    KMI_GEMM_BODY("kmi_gemm_w8a16_tiled", KIND_W8A16, true)
 }
 
 extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, const void* bias, int M, int N, int K, void* stream) {

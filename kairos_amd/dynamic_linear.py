@@ -76,9 +76,9 @@ class DynamicLinear(torch.nn.Module):
     def _tileable(self):
         return self.tiled_weights and self.out_features % 128 == 0
 
-    def _converted(self, fmt):
+    def _converted(self, fmt, tiled=None):
         """int8 or fp16 copy of the weight in the temp cache; converts only if it is not there."""
-        tiled = self._tileable()
+        tiled = self._tileable() if tiled is None else tiled
         dtype = torch.int8 if fmt == 'i8' else torch.float16
         buf, hit = self._cache().get(self._uid, (fmt, tiled), self.shape, dtype, self.qweight.device)
         if not hit:
@@ -124,8 +124,8 @@ class DynamicLinear(torch.nn.Module):
             out = torch.empty((m, N), device=x.device, dtype=torch.float16)
             ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
         elif comp_type in (_W8A16_GEMM, _W8A16_GEMV):
-            w8, tiled = self._converted('i8')
-            out = ops.w8a16_gemm_forward(x, w8, self.scales_1, N, bias=self.bias, tiled=tiled)
+            w8, _ = self._converted('i8', tiled=False)       # this lane widens int8 in registers: row-major source
+            out = ops.w8a16_gemm_forward(x, w8, self.scales_1, N, bias=self.bias)
         elif comp_type == _FP16:
             w16, tiled = self._converted('f16')
             out = ops.f16_gemm_forward(x, w16, N, bias=self.bias, tiled=tiled)

@@ -134,13 +134,13 @@ def w8a8_gemm_acc_i32(in_feats, kernel, N):
     return acc
 
 
-def w8a16_gemm_forward(x, w8, wscales, N, bias=None, tiled=False):
-    """fp16 [M, N] <- fp16 [M, K] x int8 [N, K], per-channel scale in the epilogue."""
+def w8a16_gemm_forward(x, w8, wscales, N, bias=None):
+    """fp16 [M, N] <- fp16 [M, K] x int8 [N, K] (row-major), per-channel scale in the epilogue."""
     _need(x, torch.float16, "x"); _need(w8, torch.int8, "w8")
     x2 = _flat2d(x)
     M, K = x2.shape
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
-    fn = _lib.load().kmi_gemm_w8a16_tiled if tiled else _lib.load().kmi_gemm_w8a16
+    fn = _lib.load().kmi_gemm_w8a16
     _call("gemm_w8a16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w8.data_ptr(), wscales.data_ptr(), _ptr(bias),
           M, N, K, _stream())
     return out

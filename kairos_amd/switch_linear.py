@@ -25,7 +25,12 @@ class SwitchLinear(DynamicLinear):
         q.ori_weight = torch.empty(q.shape, dtype=torch.float16, device=device)
         ops.dequant_interleaved_int4_to_fp16(q.ori_weight, q.qweight, q.scales, q.scaled_zeros, 128, tiled=tiled)
         q._resident_tiled = tiled
+        if tiled:       # the W8A16 lane reads row-major int8
+            q.smq_weight_rowmajor = torch.empty(q.shape, dtype=torch.int8, device=device)
+            ops.dequant_interleaved_int4_to_int8(q.smq_weight_rowmajor, q.qweight, q.scales_to8, q.scaled_zeros_to8, 128)
         return q
 
-    def _converted(self, fmt):
+    def _converted(self, fmt, tiled=None):
+        if fmt == 'i8' and tiled is False and self._resident_tiled:
+            return self.smq_weight_rowmajor, False
         return (self.smq_weight if fmt == 'i8' else self.ori_weight), self._resident_tiled

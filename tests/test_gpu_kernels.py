@@ -268,15 +268,13 @@ def test_gemm_tiled_operands_match_row_major(ops, tile):
     try:
         a = ops.f16_gemm_forward(xd, dev(p["w16"]), N)
         b = ops.f16_gemm_forward(xd, t16, N, tiled=True)
-        c = ops.w8a16_gemm_forward(xd, dev(p["w8"]), s1, N)
-        d = ops.w8a16_gemm_forward(xd, t8, s1, N, tiled=True)
         e = torch.empty((M, N), dtype=torch.float16, device="cuda")
         f = torch.empty((M, N), dtype=torch.float16, device="cuda")
         ops.w8a8_gemm_forward(a8, dev(p["w8"]), s1, sx, e)
         ops.w8a8_gemm_forward(a8, t8, s1, sx, f, tiled=True)
     finally:
         ops.force_gemm_tile(0)
-    assert torch.equal(a, b) and torch.equal(c, d) and torch.equal(e, f)
+    assert torch.equal(a, b) and torch.equal(e, f)
 
 
 def test_gemm_bias(ops):
