@@ -424,7 +424,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: feeds M0
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
@@ -442,8 +442,13 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     // ---- global sources.  Load i of wave w fills the KiB region R = 4*i + w = rows 16R .. 16R+15.
-    const char* src[NLD];
-    long step[NLD];
+    // Addresses are a wave-uniform base (advanced per k-stage with scalar adds) plus a per-lane
+    // 32-bit offset that never changes, so the loop carries no vector address arithmetic.
+    const char* a_base = static_cast<const char*>(p.a);
+    const char* b_base = static_cast<const char*>(p.b);
+    if constexpr (TILED_B) b_base += (long)(n0 / KMI_TILE_N) * T * (KMI_TILE_N * 64);
+    constexpr long B_STEP = TILED_B ? KMI_TILE_N * 64 : 64;
+    uint32_t voff[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int row = 16 * (4 * i + wave) + (lane >> 2);
@@ -452,31 +457,30 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
         if (16 * (4 * i) < BM) {                             // region lies in the A part (BM % 64 == 0)
             int m = m0 + row;
             m = m < M ? m : M - 1;
-            src[i] = static_cast<const char*>(p.a) + (long)m * row_bytes + c * 16;
-            step[i] = 64;
+            voff[i] = (uint32_t)((long)m * row_bytes + c * 16);
         } else if constexpr (TILED_B) {
             const int rb = row - BM;
             int strip = rb >> 7;
             if (n0 + strip * KMI_TILE_N >= N) strip = 0;
-            src[i] = static_cast<const char*>(p.b) + ((long)(n0 / KMI_TILE_N) + strip) * T * (KMI_TILE_N * 64) +
-                     (rb & 127) * 64 + pc * 16;
-            step[i] = KMI_TILE_N * 64;
+            voff[i] = (uint32_t)((long)strip * T * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
         } else {
             int n = n0 + row - BM;
             n = n < N ? n : N - 1;
-            src[i] = static_cast<const char*>(p.b) + (long)n * row_bytes + c * 16;
-            step[i] = 64;
+            voff[i] = (uint32_t)((long)n * row_bytes + c * 16);
         }
     }
     auto issue_stage = [&](int t) {                          // k-stage t -> LDS stage t % NS
         const int tt = t < T ? t : T - 1;                    // past the end: harmless reload into a free stage
         char* dst = smem + (t % NS) * STAGE + wave * 1024;
+        const char* ab = a_base + (long)tt * 64;
+        const char* bb = b_base + (long)tt * B_STEP;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
 #ifdef KMI_DBG_NOLOAD
             if (t >= NS) continue;
 #endif
-            __builtin_amdgcn_global_load_lds((global_void_ptr)(src[i] + tt * step[i]), (lds_void_ptr)(dst + i * 4096), 16, 0, 0);
+            const char* g = ((16 * (4 * i) < BM) ? ab : bb) + voff[i];
+            __builtin_amdgcn_global_load_lds((global_void_ptr)g, (lds_void_ptr)(dst + i * 4096), 16, 0, 0);
         }
     };
 
@@ -609,6 +613,8 @@ static int gemm_check(const char* fn, const GemmArgs& a, bool tiled) {
     if (a.M < 0 || a.N <= 0 || a.K <= 0 || (a.K & 127) || (a.N & 3))
         return kmi_set_error(KMI_E_SHAPE, "%s: need M>=0, N%%4==0, K%%128==0 (M=%d N=%d K=%d)", fn, a.M, a.N, a.K);
     if (tiled && (a.N % KMI_TILE_N)) return kmi_set_error(KMI_E_SHAPE, "%s: tiled operand needs N%%%d==0 (N=%d)", fn, KMI_TILE_N, a.N);
+    if ((long)a.M * a.K * 2 >= (1L << 32) || (long)a.N * a.K * 2 >= (1L << 32))
+        return kmi_set_error(KMI_E_SHAPE, "%s: an operand of 4 GiB or more is not supported (M=%d N=%d K=%d)", fn, a.M, a.N, a.K);
     return KMI_OK;
 }
 
