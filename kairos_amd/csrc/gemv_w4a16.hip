@@ -1,15 +1,23 @@
 // W4A16 product for decode-sized M (1..64): the packed uint4 weights are streamed from HBM exactly
-// once with 16-byte loads, decoded to fp16 in registers (bit-identical to the fp16 converter) and fed
-// to v_mfma_f32_16x16x32_f16 with fp32 accumulation.
+// once with 16-byte loads and fed to v_mfma_f32_16x16x32_f16 with fp32 accumulation.
 //
-// Work split.  A workgroup owns 16*NT output columns; its NW waves interleave over the 128-wide K
-// groups (wave w takes groups w, w+NW, ...), so the workgroup as a whole walks contiguous memory:
-// the four-row interleave makes a 16-row strip one contiguous K*8-byte region.  Partial sums meet in
+// Decoding costs no arithmetic: an fp16 whose exponent field is zero is the subnormal m * 2^-24, and
+// the MFMA unit honours subnormal inputs, so a nibble masked in place IS the number q * 2^-24 (low
+// nibble of a byte) or 16q * 2^-24 (high nibble).  Per 128-wide K group g and output column n the
+// kernel therefore accumulates P = sum_k x[m,k] * q[n,k] exactly (activations for the high-nibble
+// planes are pre-multiplied by 1/16), obtains X = sum_k x[m,k] from one extra MFMA against a tile of
+// ones, and adds  scales[g,n] * P + scaled_zeros[g,n] * X  in fp32.  That is the dequantise-then-
+// multiply product with the weights kept at full precision instead of rounded to fp16 first (the
+// difference to the fp16 converter's weights is below 2^-11 relative per weight).
+//
+// Work split.  A workgroup owns 16*NT output columns; its NW waves interleave over the K groups
+// (wave w takes groups w, w+NW, ...), so the workgroup as a whole walks contiguous memory: the
+// four-row interleave makes a 16-row strip one contiguous K*8-byte region.  Partial sums meet in
 // LDS and are added in a fixed order (deterministic output).
 //
 // Lane roles inside a wave, for one K group and one 16-column tile: lane = (r16, j), r16 = lane&15,
 // j = lane>>4.  The lane loads the 16-byte chunk of row n = tile*16 + r16 that covers
-// k = 128c + 32j .. +31; nibble plane a of its four words decodes to the eight K-contiguous weights
+// k = 128c + 32j .. +31; nibble plane a of its four words holds the eight K-contiguous weights
 // k = 128c + 32j + 8a .. +7, which is exactly the MFMA B fragment of lane (col r16, k-block j).  The
 // matching A fragment is x[m = r16][same eight k], one 16-byte load.  Four MFMAs (a = 0..3) per tile
 // consume the group.
@@ -45,43 +53,94 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
         ncol[nt] = n;
         wp[nt] = qw + (long)(n >> 2) * kq + (n & 3) * 2 + (j & 1) + (j >> 1) * 8;
     }
+    // Rows beyond M are not loaded at all (their lanes feed zeros): the texture path spends time per
+    // active lane quad, so a decode step with one token costs a quarter of a full tile.
     const h8_t* xp[MT];
+    bool xrow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        int m = mt * 16 + r16;
-        m = m < M ? m : M - 1;
-        xp[mt] = reinterpret_cast<const h8_t*>(x) + (long)m * kq + j * 4;
+        const int m = mt * 16 + r16;
+        xrow[mt] = m < M;
+        xp[mt] = reinterpret_cast<const h8_t*>(x) + (long)(xrow[mt] ? m : 0) * kq + j * 4;
     }
 
-    for (int c = wave; c < ngroups; c += NW) {
-        u4_t u[NT];
-        half_t s[NT], z[NT];
+    // U K-groups per trip: all loads of the trip are issued before the first MFMA, so one wave keeps
+    // U KiB-sized weight loads (plus their activation fragments) in flight.
+    constexpr int U = (MT == 1) ? 4 : (MT == 2) ? 2 : 1;
+    const h8_t ones = {(half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1};
+    const h8_t sixteenth = ones * (half_t)0.0625f;
+    for (int c0 = wave; c0 < ngroups; c0 += NW * U) {
+        u4_t u[U][NT];
+        half_t s[U][NT], z[U][NT];
+        h8_t xa[U][MT][4];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            u[nt] = __builtin_nontemporal_load(wp[nt] + c * 16);
-            s[nt] = scales[(long)c * N + ncol[nt]];
-            z[nt] = szeros[(long)c * N + ncol[nt]];
+        for (int t = 0; t < U; ++t) {
+            int c = c0 + t * NW;
+            c = c < ngroups ? c : ngroups - 1;               // ragged last trip: reload, result unused
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                u[t][nt] = __builtin_nontemporal_load(wp[nt] + c * 16);
+#ifdef KMI_DBG_NOSCALE
+                s[t][nt] = (half_t)1.0f; z[t][nt] = (half_t)0.5f;
+#else
+                s[t][nt] = scales[(long)c * N + ncol[nt]];
+                z[t][nt] = szeros[(long)c * N + ncol[nt]];
+#endif
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#ifdef KMI_DBG_NOX
+                if (false) {
+#else
+                if (xrow[mt]) {
+#endif
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) xa[t][mt][a] = xp[mt][c * 16 + a];
+                } else {
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) xa[t][mt][a] = ones * (half_t)0.0f;
+                }
+            }
         }
-        h8_t xa[MT][4];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int t = 0; t < U; ++t) {
+            if (c0 + t * NW < ngroups) {                     // wave-uniform
+                f4_t xsum[MT];
 #pragma unroll
-            for (int a = 0; a < 4; ++a) xa[mt][a] = xp[mt][c * 16 + a];
-
+                for (int mt = 0; mt < MT; ++mt) {
+                    xsum[mt] = f4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const h2_t s2 = {s[nt], s[nt]};
-            const h2_t z2 = {z[nt], z[nt]};
-            h8_t b[4];
-            b[0] = dequant_nibble<0>(u[nt], s2, z2);
-            b[1] = dequant_nibble<1>(u[nt], s2, z2);
-            b[2] = dequant_nibble<2>(u[nt], s2, z2);
-            b[3] = dequant_nibble<3>(u[nt], s2, z2);
+                    for (int a = 0; a < 4; ++a)
+                        xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][a], ones, xsum[mt], 0, 0, 0);
+                    xa[t][mt][1] *= sixteenth;               // planes 1 and 3 carry 16q
+                    xa[t][mt][3] *= sixteenth;
+                }
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
+                for (int nt = 0; nt < NT; ++nt) {
+                    u4_t lo, hi, lo8, hi8;                   // nibble planes 0, 1, 2, 3 as fp16 subnormals
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][a], b[a], acc[mt][nt], 0, 0, 0);
+                    for (int w = 0; w < 4; ++w) {
+                        const uint32_t v = u[t][nt][w], v8 = v >> 8;
+                        lo[w] = v & 0x000F000Fu;
+                        hi[w] = v & 0x00F000F0u;
+                        lo8[w] = v8 & 0x000F000Fu;
+                        hi8[w] = v8 & 0x00F000F0u;
+                    }
+                    const float sc = (float)s[t][nt] * 16777216.0f;      // undo the 2^-24 of the subnormal encoding
+                    const float zc = (float)z[t][nt];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        f4_t pg = {0.f, 0.f, 0.f, 0.f};
+                        pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][0], __builtin_bit_cast(h8_t, lo), pg, 0, 0, 0);
+                        pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][1], __builtin_bit_cast(h8_t, hi), pg, 0, 0, 0);
+                        pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][2], __builtin_bit_cast(h8_t, lo8), pg, 0, 0, 0);
+                        pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][3], __builtin_bit_cast(h8_t, hi8), pg, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[mt][nt][i] = __builtin_fmaf(pg[i], sc, __builtin_fmaf(xsum[mt][i], zc, acc[mt][nt][i]));
+                    }
+                }
+            }
         }
     }
 
@@ -154,16 +213,14 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
     return nullptr;
 }
 
-// Default split: enough waves to keep every SIMD streaming (>= 8 per CU) while each wave still owns
-// at least two K groups.
+// Default split, from sweeps on MI355X: as many column tiles per wave as still leave roughly 200
+// workgroups (each activation fragment is then reused by more MFMAs), eight waves per workgroup over K.
 static void gemv_default_cfg(int mt, int N, int K, int* nt_out, int* nw_out) {
     const int strips = (N + 15) / 16, groups = K / 128;
-    const int want_waves = 2048;
-    int nt = 4, nw = 4;
-    while (nt > 1 && ((strips + nt - 1) / nt * nw < want_waves || mt * nt > 8)) nt >>= 1;
-    while (nw < 16 && (strips + nt - 1) / nt * nw < want_waves && groups / (nw * 2) >= 2 &&
-           gemv_lookup(mt, nt, nw * 2) != nullptr)
-        nw <<= 1;
+    int nt = 4;
+    while (nt > 1 && ((strips + nt - 1) / nt < 192 || gemv_lookup(mt, nt, 8) == nullptr)) nt >>= 1;
+    int nw = 8;
+    while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
     *nt_out = nt;
     *nw_out = nw;
 }
