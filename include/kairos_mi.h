@@ -21,6 +21,7 @@
 #ifndef KAIROS_MI_H
 #define KAIROS_MI_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -127,6 +128,15 @@ int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, 
 void kmi_gemm_force_tile(int tile);
 /* The workgroup tile (64, 128 or 256 rows) the automatic choice uses for an M x N output. */
 int kmi_gemm_pick_tile(int M, int N);
+
+/* Optional scratch for split-K (used when the output tiles alone cannot fill the GPU, i.e. mid-sized
+ * M): the calling thread registers a caller-owned device buffer; GEMM calls made by that thread then
+ * write fp32/int32 partial sums there and reduce them with a second kernel on the same stream, in a
+ * fixed order (deterministic).  The buffer must outlive those calls; calls that share it must be
+ * ordered on one stream.  ptr = NULL unregisters.  No reference counterpart. */
+int kmi_gemm_set_workspace(void* ptr, size_t bytes);
+/* Tuning hook for the calling thread: 0 = automatic split count, else the number of K splits. */
+void kmi_gemm_force_splits(int splits);
 
 /* ---- interval lookup table (host only) --------------------------------------------------------- */
 

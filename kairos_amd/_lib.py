@@ -33,6 +33,8 @@ SIGNATURES = {
     "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_force_tile": [_I],
     "kmi_gemm_pick_tile": [_I, _I],
+    "kmi_gemm_set_workspace": [_P, ctypes.c_size_t],
+    "kmi_gemm_force_splits": [_I],
     "kmi_lut_new": [],
     "kmi_lut_free": [_P],
     "kmi_lut_record": [_P, _I, _I],
@@ -41,7 +43,7 @@ SIGNATURES = {
     "kmi_lut_size": [_P],
 }
 _RESTYPE = {"kmi_get_last_error_string": ctypes.c_char_p, "kmi_lut_new": _P, "kmi_lut_free": None,
-            "kmi_gemm_force_tile": None}
+            "kmi_gemm_force_tile": None, "kmi_gemm_force_splits": None}
 
 _lib = None
 

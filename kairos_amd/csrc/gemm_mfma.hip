@@ -25,6 +25,8 @@ struct GemmArgs {
     const half_t* ascales;    // W8A8: [M]
     const half_t* bias;       // [N] or null
     int M, N, K;
+    void* partial;            // split-K: [splits][M][N] fp32 / int32 partial sums, else null
+    int splits;               // number of K splits (1 = none)
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
@@ -36,6 +38,82 @@ __device__ __forceinline__ void i8x4_to_h2x2(uint32_t w, h2_t& lo, h2_t& hi) {
     const uint32_t u = w ^ 0x80808080u;
     lo = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - k1152;
     hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - k1152;
+}
+
+// Split-K: a workgroup that only covers part of K writes its raw accumulators (fp32 or int32, 4 bytes
+// each) to slice `split` of the partial buffer; splitk_reduce_kernel adds the slices in a fixed order
+// and applies the epilogue arithmetic.  Lane layout as in gemm_epilogue below.
+template <int BM, int BN, int FM, int FN, typename acc_t>
+__device__ __forceinline__ void store_partial(const GemmArgs& p, acc_t (&acc)[FM][FN], int split, int m0, int n0,
+                                              int wave, int lane) {
+    const int M = p.M, N = p.N;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int c = lane & 31, hl = lane >> 5;
+    const int mw = m0 + wm * (BM / 2), nw = n0 + wn * (BN / 2);
+    uint32_t* dst = static_cast<uint32_t*>(p.partial) + (long)split * M * N;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = mw + i * 32 + c;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nw + j * 32 + 8 * g + 4 * hl;       // four consecutive columns, N % 4 == 0
+                if (m < M && n < N) {
+                    u4_t v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const auto elem = acc[i][j][4 * g + r];          // copy out of the vector first:
+                        v[r] = __builtin_bit_cast(uint32_t, elem);       // bit_cast needs an addressable scalar
+                    }
+                    *reinterpret_cast<u4_t*>(dst + (long)m * N + n) = v;
+                }
+            }
+    }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
+    const long quad = (long)blockIdx.x * 256 + threadIdx.x;       // one thread = four consecutive columns
+    const long total = (long)p.M * p.N / 4;
+    if (quad >= total) return;
+    const long e0 = quad * 4;
+    const int m = (int)(e0 / p.N), n = (int)(e0 - (long)m * p.N);
+    constexpr bool I8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
+    int isum[4] = {0, 0, 0, 0};
+    float fsum[4] = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t* part = static_cast<const uint32_t*>(p.partial);
+    for (int s = 0; s < p.splits; ++s) {
+        const u4_t v = *reinterpret_cast<const u4_t*>(part + (long)s * p.M * p.N + e0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t w = v[r];                         // scalar copy: bit_cast of a vector element misreads
+            if constexpr (I8) isum[r] += (int)w;
+            else fsum[r] += __builtin_bit_cast(float, w);
+        }
+    }
+    if constexpr (KIND == KIND_W8A8_ACC) {
+        int* o = static_cast<int*>(p.out) + e0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = isum[r];
+    } else {
+        half_t h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v;
+            if constexpr (KIND == KIND_W8A8) {
+                v = (float)isum[r] * ((float)p.wscales[n + r] * (float)p.ascales[m]);
+                asm volatile("" : "+v"(v));                  // two roundings, as in gemm_epilogue
+            } else if constexpr (KIND == KIND_W8A16) {
+                v = fsum[r] * (float)p.wscales[n + r];
+            } else {
+                v = fsum[r];
+            }
+            h[r] = (half_t)v;
+            if (p.bias) h[r] = (half_t)((float)h[r] + (float)p.bias[n + r]);
+        }
+        *reinterpret_cast<h4_t*>(static_cast<half_t*>(p.out) + e0) = h4_t{h[0], h[1], h[2], h[3]};
+    }
 }
 
 // Epilogue shared by both kernels.  The MFMAs are issued with the weight fragment as the first
@@ -199,10 +277,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
-    tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    const int TM_ = (M + BM - 1) / BM, TN_ = (N + BN - 1) / BN;
+    const int split = blockIdx.x / (TM_ * TN_);
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const long a_row_bytes = I8 ? (long)K : (long)K * 2;
-    const int KT = (int)(a_row_bytes >> 7);
+    const int KT_all = (int)(a_row_bytes >> 7);
+    const int kt_per = (KT_all + p.splits - 1) / p.splits;
+    const int kt0 = split * kt_per;                          // this workgroup covers k-tiles kt0 .. kt0+KT-1
+    const int KT = (kt0 + kt_per <= KT_all) ? kt_per : KT_all - kt0;
 
     acc_t acc[FM][FN];
 #pragma unroll
@@ -258,13 +341,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
     auto load_tile = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u4_t*>(pa[i] + (long)kt * 128);
+        for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u4_t*>(pa[i] + (long)(kt0 + kt) * 128);
 #pragma unroll
         for (int i = 0; i < B_CH; ++i) {
-            rb[i] = *reinterpret_cast<const u4_t*>(pb[i] + (long)kt * b_step);
+            rb[i] = *reinterpret_cast<const u4_t*>(pb[i] + (long)(kt0 + kt) * b_step);
             if constexpr (KIND == KIND_W4A16) {
-                rs[i] = p.scales[(long)(kt >> 1) * N + scale_col[i]];
-                rz[i] = p.szeros[(long)(kt >> 1) * N + scale_col[i]];
+                rs[i] = p.scales[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
+                rz[i] = p.szeros[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
             }
         }
     };
@@ -388,7 +471,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     }
 
     __syncthreads();                                         // staging LDS is reused by the epilogue
-    if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+    if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
+    else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
 }
 
@@ -428,10 +512,15 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
-    tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    const int TM_ = (M + BM - 1) / BM, TN_ = (N + BN - 1) / BN;
+    const int split = blockIdx.x / (TM_ * TN_);
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const long row_bytes = I8 ? (long)K : (long)K * 2;
-    const int T = (int)(row_bytes >> 6);                    // 64-byte stages along K
+    const int T_all = (int)(row_bytes >> 6);                // 64-byte stages along K
+    const int t_per = (T_all + p.splits - 1) / p.splits;
+    const int t0 = split * t_per;                            // this workgroup covers stages t0 .. t0+T-1
+    const int T = (t0 + t_per <= T_all) ? t_per : T_all - t0;
 
     acc_t acc[FM][FN];
 #pragma unroll
@@ -446,7 +535,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     // 32-bit offset that never changes, so the loop carries no vector address arithmetic.
     const char* a_base = static_cast<const char*>(p.a);
     const char* b_base = static_cast<const char*>(p.b);
-    if constexpr (TILED_B) b_base += (long)(n0 / KMI_TILE_N) * T * (KMI_TILE_N * 64);
+    if constexpr (TILED_B) b_base += (long)(n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64);
     constexpr long B_STEP = TILED_B ? KMI_TILE_N * 64 : 64;
     uint32_t voff[NLD];
 #pragma unroll
@@ -462,7 +551,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
             const int rb = row - BM;
             int strip = rb >> 7;
             if (n0 + strip * KMI_TILE_N >= N) strip = 0;
-            voff[i] = (uint32_t)((long)strip * T * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
+            voff[i] = (uint32_t)((long)strip * T_all * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
         } else {
             int n = n0 + row - BM;
             n = n < N ? n : N - 1;
@@ -470,7 +559,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
         }
     }
     auto issue_stage = [&](int t) {                          // k-stage t -> LDS stage t % NS
-        const int tt = t < T ? t : T - 1;                    // past the end: harmless reload into a free stage
+        const int tt = t0 + (t < T ? t : T - 1);             // past the end: harmless reload into a free stage
         char* dst = smem + (t % NS) * STAGE + wave * 1024;
         const char* ab = a_base + (long)tt * 64;
         const char* bb = b_base + (long)tt * B_STEP;
@@ -561,13 +650,49 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #undef KMI_STAGE_BARRIER
 
-    if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+    if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
+    else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
+// Caller-owned scratch for split-K partial sums, registered per host thread.  Optional: without it
+// (or when it is too small) no split is used.
+static thread_local void* g_workspace = nullptr;
+static thread_local size_t g_workspace_bytes = 0;
+extern "C" int kmi_gemm_set_workspace(void* ptr, size_t bytes) {
+    if (ptr && !kmi_aligned16(ptr)) return kmi_set_error(KMI_E_ALIGN, "kmi_gemm_set_workspace: pointer must be 16-byte aligned");
+    g_workspace = ptr;
+    g_workspace_bytes = ptr ? bytes : 0;
+    return KMI_OK;
+}
+static thread_local int g_force_splits = 0;
+extern "C" void kmi_gemm_force_splits(int splits) { g_force_splits = splits; }
+
+// Number of K splits: only when the output tiles alone cannot occupy the chip, every split keeps at
+// least four 128-byte k-tiles, and the partial sums fit the registered workspace.
+static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
+    const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    int s = 1;
+    if (g_force_splits > 0) s = g_force_splits;
+    else if (tiles < 256) {
+        s = (int)(512 / tiles);
+        if (s > 8) s = 8;
+    }
+    if (s > ktiles / 4) s = ktiles / 4;
+    const size_t per = (size_t)M * N * 4;
+    if (per == 0 || g_workspace == nullptr) return 1;
+    if ((size_t)s * per > g_workspace_bytes) s = (int)(g_workspace_bytes / per);
+    if (s > 1) {                                              // no empty split
+        const int per_split = (ktiles + s - 1) / s;
+        s = (ktiles + per_split - 1) / per_split;
+    }
+    return s < 2 ? 1 : s;
+}
+
 template <int KIND, int BM, int BN, bool TILED>
-static int launch_gemm(const GemmArgs& a, hipStream_t st) {
+static int launch_gemm(const GemmArgs& a_in, hipStream_t st) {
+    GemmArgs a = a_in;
     constexpr bool DIRECT = (KIND == KIND_F16 || KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     constexpr int NS = 4;
     constexpr size_t lds = DIRECT ? (size_t)NS * (BM + BN) * 64 : 2 * (size_t)(BM + BN) * 128;
@@ -582,8 +707,17 @@ static int launch_gemm(const GemmArgs& a, hipStream_t st) {
             raised = true;
         }
     }
-    const dim3 grid(((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM)), block(256);
+    const bool i8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
+    // units the kernels split K in: 128-byte k-tiles (register-staged) or 64-byte stages (direct)
+    const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
+    a.splits = pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units);
+    a.partial = a.splits > 1 ? g_workspace : nullptr;
+    const dim3 grid(((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
+    if (a.splits > 1) {
+        const long quads = (long)a.M * a.N / 4;
+        hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, a);
+    }
     return KMI_OK;
 }
 
@@ -633,42 +767,42 @@ extern "C" int kmi_gemm_w4a16(void* out, const void* x, const void* qweight, con
                               const void* bias, int M, int N, int K, int G, void* stream) {
     if (G != 128) return kmi_set_error(KMI_E_GROUP, "kmi_gemm_w4a16: group size %d unsupported (128 only)", G);
     if (!scales || !szeros) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w4a16: NULL scale table");
-    GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_w4a16", KIND_W4A16, false)
 }
 
 extern "C" int kmi_gemm_w8a16(void* out, const void* x, const void* w8, const void* wscales, const void* bias,
                               int M, int N, int K, void* stream) {
     if (!wscales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a16: NULL wscales");
-    GemmArgs a{out, x, w8, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, x, w8, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_w8a16", KIND_W8A16, false)
 }
 
 extern "C" int kmi_gemm_w8a8(void* out, const void* a8, const void* w8, const void* wscales, const void* ascales,
                              const void* bias, int M, int N, int K, void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8: NULL scale vector");
-    GemmArgs a{out, a8, w8, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, a8, w8, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_w8a8", KIND_W8A8, false)
 }
 
 extern "C" int kmi_gemm_w8a8_acc_i32(void* acc, const void* a8, const void* w8, int M, int N, int K, void* stream) {
-    GemmArgs a{acc, a8, w8, nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K};
+    GemmArgs a{acc, a8, w8, nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_w8a8_acc_i32", KIND_W8A8_ACC, false)
 }
 
 extern "C" int kmi_gemm_f16(void* out, const void* x, const void* w16, const void* bias, int M, int N, int K, void* stream) {
-    GemmArgs a{out, x, w16, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, x, w16, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_f16", KIND_F16, false)
 }
 
 extern "C" int kmi_gemm_w8a8_tiled(void* out, const void* a8, const void* w8t, const void* wscales, const void* ascales,
                                    const void* bias, int M, int N, int K, void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8_tiled: NULL scale vector");
-    GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_w8a8_tiled", KIND_W8A8, true)
 }
 
 extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, const void* bias, int M, int N, int K, void* stream) {
-    GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K};
+    GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
     KMI_GEMM_BODY("kmi_gemm_f16_tiled", KIND_F16, true)
 }

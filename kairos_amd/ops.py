@@ -105,6 +105,8 @@ def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZ
 
 def gemm_forward(x, qweight, scales, scaled_zeros, bias=None):
     """W4A16 MFMA GEMM for any m (gemm_cuda.cu:1126-1235).  Returns fp16 [*x.shape[:-1], N]."""
+    if _workspace is None:
+        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
     N, K = qweight.shape[0] * 4, qweight.shape[1]
     x2 = _flat2d(x)
@@ -117,6 +119,8 @@ def gemm_forward(x, qweight, scales, scaled_zeros, bias=None):
 
 def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, tiled=False):
     """out_feats fp16 [M, N] <- int8 [M, K] x int8 [N, K] (w8a8_gemm_cuda.cu:909-954)."""
+    if _workspace is None:
+        ensure_workspace(device=in_feats.device)
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel"); _need(out_feats, torch.float16, "out_feats")
     M, K = in_feats.shape
     N = out_feats.shape[-1]
@@ -127,6 +131,8 @@ def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, 
 
 def w8a8_gemm_acc_i32(in_feats, kernel, N):
     """Raw int32 accumulators [M, N] of the W8A8 product."""
+    if _workspace is None:
+        ensure_workspace(device=in_feats.device)
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel")
     M, K = in_feats.shape
     acc = torch.empty((M, N), dtype=torch.int32, device=in_feats.device)
@@ -136,6 +142,8 @@ def w8a8_gemm_acc_i32(in_feats, kernel, N):
 
 def w8a16_gemm_forward(x, w8, wscales, N, bias=None):
     """fp16 [M, N] <- fp16 [M, K] x int8 [N, K] (row-major), per-channel scale in the epilogue."""
+    if _workspace is None:
+        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(w8, torch.int8, "w8")
     x2 = _flat2d(x)
     M, K = x2.shape
@@ -148,6 +156,8 @@ def w8a16_gemm_forward(x, w8, wscales, N, bias=None):
 
 def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
     """fp16 [M, N] <- fp16 [M, K] x fp16 [N, K] (`input @ tmp_weight.T`, dynamic_linear.py:163)."""
+    if _workspace is None:
+        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(w16, torch.float16, "w16")
     x2 = _flat2d(x)
     M, K = x2.shape
@@ -160,6 +170,29 @@ def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
 def gemm_tile_for(M, N):
     """Workgroup tile (64/128/256) the automatic choice uses for an M x N output."""
     return _lib.load().kmi_gemm_pick_tile(int(M), int(N))
+
+
+_workspace = None
+
+
+def ensure_workspace(nbytes=64 << 20, device="cuda"):
+    """Registers a persistent split-K scratch buffer (once per process) with the library."""
+    global _workspace
+    if _workspace is None or _workspace.numel() < nbytes:
+        _workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _lib.check(_lib.load().kmi_gemm_set_workspace(_workspace.data_ptr(), _workspace.numel()))
+    return _workspace
+
+
+def drop_workspace():
+    global _workspace
+    _lib.check(_lib.load().kmi_gemm_set_workspace(None, 0))
+    _workspace = None
+
+
+def force_gemm_splits(splits):
+    """Tuning hook: 0 = automatic, else the number of K splits (needs a registered workspace)."""
+    _lib.load().kmi_gemm_force_splits(int(splits))
 
 
 def force_gemm_tile(tile):

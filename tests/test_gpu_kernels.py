@@ -237,12 +237,14 @@ def test_gemm_w4a16_f16_w8a16(ops, M, tile):
     ref = O.gemm_f16(x, p["w16"])
     xd = dev(x)
     ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(1)                                # one workgroup per tile walks all of K
     try:
         out4 = ops.gemm_forward(xd, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]))
         out16 = ops.f16_gemm_forward(xd, dev(p["w16"]), N)
         out816 = ops.w8a16_gemm_forward(xd, dev(p["w8"]), dev(p["scales_1"]), N)
     finally:
         ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
     assert O.max_abs_rel(host(out4), ref) < 2e-3
     assert O.max_abs_rel(host(out16), ref) < 2e-3
     assert torch.equal(out4, out16)                         # same fp16 weights, same accumulation order
@@ -275,6 +277,39 @@ def test_gemm_tiled_operands_match_row_major(ops, tile):
     finally:
         ops.force_gemm_tile(0)
     assert torch.equal(a, b) and torch.equal(e, f)
+
+
+@pytest.mark.parametrize("splits", [2, 3, 4])
+@pytest.mark.parametrize("tile", [64, 128])
+def test_gemm_split_k(ops, tile, splits):
+    """K split over several workgroups with the partial sums reduced in a second kernel: the int8 lane
+    stays bit-exact (integer partials), the fp16 lanes stay within tolerance and deterministic."""
+    N, K, M = 256, 2048, 100
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=9)
+    xd = dev(x)
+    ref = O.gemm_f16(x, p["w16"])
+    a8_ref, sx_ref = O.quant_act_i8(x)
+    ops.ensure_workspace()
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(splits)
+    try:
+        out4 = ops.gemm_forward(xd, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]))
+        again = ops.gemm_forward(xd, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]))
+        out16 = ops.f16_gemm_forward(xd, dev(p["w16"]), N)
+        out816 = ops.w8a16_gemm_forward(xd, dev(p["w8"]), dev(p["scales_1"]), N)
+        acc = ops.w8a8_gemm_acc_i32(dev(a8_ref), dev(p["w8"]), N)
+        out88 = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        ops.w8a8_gemm_forward(dev(a8_ref), dev(p["w8"]), dev(p["scales_1"]), dev(sx_ref), out88)
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert O.max_abs_rel(host(out4), ref) < 2e-3 and torch.equal(out4, again)
+    assert O.max_abs_rel(host(out16), ref) < 2e-3
+    assert O.max_abs_rel(host(out816), O.gemm_w8a16(x, p["w8"], p["scales_1"])) < 2e-3
+    acc_ref, out_ref = O.gemm_w8a8(a8_ref, p["w8"], p["scales_1"], sx_ref)
+    assert np.array_equal(host(acc), acc_ref)
+    assert_same_bits(host(out88), out_ref)
 
 
 def test_gemm_bias(ops):
