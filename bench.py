@@ -26,6 +26,9 @@ LAYER = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), 
 M_GRID = [1 << i for i in range(13)]
 PEAK = {"hbm": 8.0e12, "f16": 2.5e15, "i8": 5.0e15}       # MI355X published: HBM3E B/s, dense MFMA op/s
 LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x")
+# HBM<->L2 bytes per launch of the dominant kernel, from the committed counter runs (profiles/
+# bench_llama3_8b_fetch_write_size.md): mean over the launches of one step, 2.0*FETCH_SIZE + WRITE_SIZE KiB.
+MEASURED_TRAFFIC = {"gemm_w8a8[256]": int((2.0 * 155660 + 130526) * 1024)}
 G = 128
 
 
@@ -141,6 +144,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-lane sweep table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is single-GPU by construction (every linear is independent; see the sharding note "
@@ -176,6 +181,13 @@ def main():
     for K in sorted({k for _, _, k in LAYER}):
         for M in M_GRID:
             acts[(M, K)] = torch.from_numpy(O.synth_acts(M, K, seed=11)).to(dev).reshape(1, M, K)
+
+    if args.calib_copy:
+        src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- lookup table -------------------------------------------------------------------------
     shapes = [(N, K) for _, N, K in LAYER]
@@ -231,7 +243,8 @@ def main():
     else:
         achieved, peak, unit, bound = dom["bytes"] / dom["sec"] / 1e9, PEAK["hbm"] / 1e9, "GB/s", "hbm"
     roofline = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                "frac": round(achieved / peak, 4), "traffic": None, "kernel": dom_label,
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(dom_label), "kernel": dom_label,
+                "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
                 "launches": dom["launches"], "avg_launch_us": round(avg_dur * 1e6, 2),
                 "share_of_kernel_time": round(dom["sec"] / total_kernel_sec, 4)}
     kernels = {k: {"launches": a["launches"], "avg_us": round(a["sec"] / a["launches"] * 1e6, 2),
