@@ -49,6 +49,7 @@ class DynamicLinear(torch.nn.Module):
         self.pre_comp_type = ''
         self.comp_type = None
         self._uid = next(_uids)     # identifies this layer's entries in the temp cache
+        self._decode_ptrs = None
         self.switch_count = 0       # times the selected lane changed between consecutive forward calls
         self.qweight = self.scales = self.scaled_zeros = None
         self.scales_to8 = self.scaled_zeros_to8 = self.scales_1 = None
@@ -93,15 +94,34 @@ class DynamicLinear(torch.nn.Module):
     @torch.no_grad()
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         shape = input.shape
-        input = input.reshape(-1, shape[-1])
-        m = input.shape[0]
+        K = shape[-1]
+        m = input.numel() // K
         if m != self.pre_m:
             self.pre_m = m
             comp = type(self).prof.get_comp_type(self.shape, m)
             if self.comp_type is not None and comp != self.comp_type:
                 self.switch_count += 1
             self.comp_type = comp
-        return self._forward(input, m, self.comp_type).reshape(*shape[:-1], -1)
+        if self.comp_type == _W4A16_GEMV and m <= ops.GEMV_MAX_M and ops._tracer is None:
+            return self._forward_decode(input, shape, m)
+        return self._forward(input.reshape(-1, K), m, self.comp_type).reshape(*shape[:-1], -1)
+
+    def _forward_decode(self, input, shape, m):
+        """Decode-sized calls are host-bound: one allocation, one C call, cached pointers."""
+        if input.dtype is not torch.float16 or not input.is_cuda or not input.is_contiguous():
+            return self._forward(input.reshape(-1, shape[-1]), m, self.comp_type).reshape(*shape[:-1], -1)
+        ptrs = self._decode_ptrs
+        if ptrs is None or ptrs[0] != self.qweight.data_ptr():
+            ptrs = self._decode_ptrs = (self.qweight.data_ptr(), self.scales.data_ptr(), self.scaled_zeros.data_ptr(),
+                                        0 if self.bias is None else self.bias.data_ptr(),
+                                        ops._lib.load().kmi_gemv_w4a16, input.device.index or 0)
+        N, K = self.shape
+        out = torch.empty(shape[:-1] + (N,), dtype=torch.float16, device=input.device)
+        rc = ptrs[4](out.data_ptr(), input.data_ptr(), ptrs[0], ptrs[1], ptrs[2], ptrs[3], m, N, K, self.group_size,
+                     ops._raw_stream(ptrs[5]) if ops._raw_stream is not None else ops._stream())
+        if rc < 0:
+            ops._lib.check(rc)
+        return out
 
     @torch.no_grad()
     def _forward(self, input: torch.Tensor, batch_token_len, comp_type) -> torch.Tensor:

@@ -31,7 +31,15 @@ def _call(name, M, N, K, fn, *args):
         _tracer.end()
 
 
+try:                                       # raw handle of torch's current stream without building a Stream object
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:                     # pragma: no cover
+    _raw_stream = None
+
+
 def _stream():
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
