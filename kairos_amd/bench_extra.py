@@ -1,0 +1,258 @@
+"""Secondary benchmarks of the switched-linear path (the headline benchmark is bench.py at the repo root).
+
+    python -m kairos_amd.bench_extra gemv70b   # decode-regime W4A16 on Llama-3-70B shapes, M = 1..32
+    python -m kairos_amd.bench_extra convert   # int4 -> int8 / fp16 / tiled conversion on Qwen2.5-7B shapes
+    python -m kairos_amd.bench_extra decoder   # random-init Llama-3-8B decoder: TTFT / TPOT / lane switches
+
+Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
+channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
+beyond the 256 MB Infinity Cache for the bandwidth-bound kernels.
+"""
+import argparse
+import json
+import math
+import sys
+import time
+
+import numpy as np
+import torch
+
+from . import ops
+from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+from .perf_profiler import Profiler
+from .temp_cache import TempCache
+from .weight_prep import prepare_linear_weight
+
+HBM = 8.0e12
+G = 128
+
+
+def _weights(N, K, seed=10):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+
+
+def _acts(M, K, seed=11):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((M, K), generator=g, dtype=torch.float32)
+    cols = torch.randperm(K, generator=g)[: int(0.01 * K)]
+    x[:, cols] *= 20.0
+    return x.to(torch.float16)
+
+
+def _time(fn, n):
+    fn(0); fn(1)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(n):
+        fn(i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / n
+
+
+def _layer(N, K, copies, dev):
+    """One prepared linear, `copies` times in distinct memory (the values do not matter for timing)."""
+    prep = {k: v.to(dev) for k, v in prepare_linear_weight(_weights(min(N, 1024), K)).items()}
+    reps = N // min(N, 1024)
+    full = {"qweight": prep["qweight"].repeat(reps, 1), "scales_1": prep["scales_1"].repeat(reps)}
+    for k in ("scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8"):
+        full[k] = prep[k].repeat(1, reps)
+    out = []
+    for c in range(copies):
+        dl = DynamicLinear(K, N, False, dev, 128)
+        for k, v in full.items():
+            setattr(dl, k, v.clone().contiguous())
+        out.append(dl)
+    return out
+
+
+def gemv70b(args):
+    """BASELINE config 3: qkv 8192->10240, gate_up 8192->57344, down 28672->8192, M = 1..32."""
+    dev = torch.device("cuda:0")
+    rows = []
+    for name, N, K in [("qkv", 10240, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)]:
+        copies = max(2, math.ceil(600e6 / (N * K / 2)))
+        layers = _layer(N, K, copies, dev)
+        for M in (1, 2, 4, 8, 16, 32):
+            x = _acts(M, K).to(dev)[None]
+            us = _time(lambda i: layers[i % copies]._forward(x, M, COMP_TYPE_NAME["w4a16_gemv"]), 40)
+            b = N * K // 2 + 4 * (K // G) * N + 2 * M * K + 2 * M * N
+            rows.append({"shape": name, "N": N, "K": K, "M": M, "us": round(us, 2), "gbps": round(b / us / 1e3, 1),
+                         "hbm_frac": round(b / us / 1e-6 / HBM, 4)})
+            print(rows[-1], file=sys.stderr, flush=True)
+        del layers
+        torch.cuda.empty_cache()
+    whole_model_gb = 80 * sum(n * k for n, k in [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]) / 2 / 1e9
+    return {"bench": "gemv70b", "unit": "us per call (event-timed, _forward incl. output allocation)", "rows": rows,
+            "whole_model_int4_gb": round(whole_model_gb, 1)}
+
+
+def convert(args):
+    """BASELINE config 4: Qwen2.5-7B shapes; int4 -> int8, fp16, tiled; temp-cache high-water mark."""
+    dev = torch.device("cuda:0")
+    shapes = [("qkv", 4608, 3584), ("gate_up", 37888, 3584), ("down", 3584, 18944)]
+    cache = TempCache()
+    rows = []
+    for name, N, K in shapes:
+        copies = max(2, math.ceil(600e6 / (N * K / 2)))
+        layers = _layer(N, K, copies, dev)
+        for dl in layers:
+            dl.temp_cache = cache
+        for fmt, es in (("i8", 1), ("f16", 2)):
+            for tiled in (False, True):
+                def call(i, fmt=fmt, tiled=tiled):
+                    cache.invalidate()
+                    layers[i % copies]._converted(fmt, tiled=tiled)
+                us = _time(call, 40)
+                b = N * K // 2 + 4 * (K // G) * N + es * N * K
+                rows.append({"shape": name, "N": N, "K": K, "to": fmt, "tiled": tiled, "us": round(us, 2),
+                             "gbps": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e-6 / HBM, 4)})
+                print(rows[-1], file=sys.stderr, flush=True)
+        del layers
+        torch.cuda.empty_cache()
+    largest = max(n * k for _, n, k in shapes) * 2
+    assert cache.peak_bytes <= largest and cache.capacity <= largest, (cache.peak_bytes, cache.capacity, largest)
+    return {"bench": "convert", "rows": rows, "temp_cache_peak_bytes": cache.peak_bytes,
+            "largest_converted_weight_bytes": largest, "temp_cache_bounded": True}
+
+
+# ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
+class _RMSNorm(torch.nn.Module):
+    def __init__(self, dim, dev):
+        super().__init__()
+        self.weight = torch.ones(dim, dtype=torch.float16, device=dev)
+
+    def forward(self, x):
+        v = x.float()
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).to(torch.float16) * self.weight
+
+
+def _rope(x, pos, theta=500000.0):
+    # x [B, H, S, D]; rotate-half formulation
+    d = x.shape[-1]
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, device=x.device, dtype=torch.float32) / d))
+    ang = pos.float()[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).to(x.dtype), torch.sin(ang).to(x.dtype)
+    x1, x2 = x[..., : d // 2], x[..., d // 2:]
+    return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
+
+
+class _Layer(torch.nn.Module):
+    def __init__(self, lin, dev, hidden=4096, heads=32, kv_heads=8):
+        super().__init__()
+        self.h, self.kv, self.d = heads, kv_heads, hidden // heads
+        self.qkv, self.o, self.gate_up, self.down = lin
+        self.n1, self.n2 = _RMSNorm(hidden, dev), _RMSNorm(hidden, dev)
+        self.k_cache = self.v_cache = None
+
+    def forward(self, x, pos0):
+        B, S, _ = x.shape
+        qkv = self.qkv(self.n1(x))
+        q, k, v = qkv.split([self.h * self.d, self.kv * self.d, self.kv * self.d], dim=-1)
+        q = q.view(B, S, self.h, self.d).transpose(1, 2)
+        k = k.view(B, S, self.kv, self.d).transpose(1, 2)
+        v = v.view(B, S, self.kv, self.d).transpose(1, 2)
+        pos = torch.arange(pos0, pos0 + S, device=x.device)
+        q, k = _rope(q, pos), _rope(k, pos)
+        if pos0 == 0:
+            self.k_cache, self.v_cache = k, v
+        else:
+            self.k_cache = torch.cat([self.k_cache, k], dim=2)
+            self.v_cache = torch.cat([self.v_cache, v], dim=2)
+        a = torch.nn.functional.scaled_dot_product_attention(q, self.k_cache, self.v_cache, is_causal=(pos0 == 0 and S > 1),
+                                                             enable_gqa=True)
+        x = x + self.o(a.transpose(1, 2).reshape(B, S, -1))
+        gu = self.gate_up(self.n2(x))
+        g, u = gu.chunk(2, dim=-1)
+        return x + self.down(torch.nn.functional.silu(g) * u)
+
+
+def decoder(args):
+    """BASELINE config 5: 32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336, vocab 128256; every linear a
+    LUT-switched DynamicLinear (fused qkv and gate_up); protocol of utils/perf_eval.py:235-275."""
+    dev = torch.device("cuda:0")
+    shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
+    prof = Profiler(shapes)
+    prof.load(args.lut)
+    DynamicLinear.prof = prof
+    nl = args.layers
+    per_shape = [_layer(N, K, nl, dev) for N, K in shapes]
+    layers = [_Layer([per_shape[s][l] for s in range(4)], dev) for l in range(nl)]
+    vocab = 128256
+    emb = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
+    head = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
+    fnorm = _RMSNorm(4096, dev)
+
+    @torch.no_grad()
+    def generate(ids, new_tokens):
+        x = emb[ids]
+        pos = 0
+        for _ in range(new_tokens):
+            h = x
+            for L in layers:
+                h = L(h, pos)
+            pos += x.shape[1]
+            logits = fnorm(h[:, -1:, :]) @ head.T
+            nxt = logits.argmax(-1)
+            x = emb[nxt]
+        torch.cuda.synchronize()
+
+    results = []
+    for B in args.batches:
+        ids = torch.randint(0, vocab, (B, args.prompt), device=dev)
+        for L in layers:
+            for lin in (L.qkv, L.o, L.gate_up, L.down):
+                lin.switch_count = 0
+        generate(ids, 2)                                                   # warm-up
+        t0 = time.perf_counter()
+        for _ in range(args.ttft_times):
+            generate(ids, 1)
+        ttft = (time.perf_counter() - t0) / args.ttft_times
+        for L in layers:
+            for lin in (L.qkv, L.o, L.gate_up, L.down):
+                lin.switch_count = 0
+        t0 = time.perf_counter()
+        generate(ids, args.new_tokens)
+        total = time.perf_counter() - t0
+        tpot = (total - ttft) / max(1, args.new_tokens - 1)
+        sw = [sum(getattr(L, n).switch_count for L in layers) / nl for n in ("qkv", "o", "gate_up", "down")]
+        results.append({"batch": B, "ttft_ms": round(ttft * 1e3, 2), "tpot_ms": round(tpot * 1e3, 3),
+                        "tokens_per_s": round(B * args.new_tokens / total, 1),
+                        "switches_per_layer": {"qkv": sw[0], "o_proj": sw[1], "gate_up": sw[2], "down": sw[3]},
+                        "prefill_lane": {n: {v: k for k, v in COMP_TYPE_NAME.items()}[prof.get_comp_type(s, B * args.prompt)]
+                                         for n, s in zip(("qkv", "o_proj", "gate_up", "down"), shapes)},
+                        "decode_lane": {n: {v: k for k, v in COMP_TYPE_NAME.items()}[prof.get_comp_type(s, B)]
+                                        for n, s in zip(("qkv", "o_proj", "gate_up", "down"), shapes)}})
+        print(results[-1], file=sys.stderr, flush=True)
+    return {"bench": "decoder", "layers": nl, "prompt": args.prompt, "new_tokens": args.new_tokens,
+            "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention and norms in PyTorch, greedy decoding",
+            "peak_hbm_gb": round(torch.cuda.max_memory_allocated() / 1e9, 2), "rows": results}
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    sub.add_parser("gemv70b")
+    sub.add_parser("convert")
+    d = sub.add_parser("decoder")
+    d.add_argument("--lut", default=None)
+    d.add_argument("--layers", type=int, default=32)
+    d.add_argument("--prompt", type=int, default=1024)
+    d.add_argument("--new-tokens", type=int, default=512)
+    d.add_argument("--ttft-times", type=int, default=3)
+    d.add_argument("--batches", type=int, nargs="+", default=[2, 4, 8, 16, 32])
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        sys.exit("bench_extra: needs a GPU (the HIP library is the only compute path)")
+    if args.cmd == "decoder" and args.lut is None:
+        import os
+        args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
+    ops.ensure_workspace()
+    res = {"gemv70b": gemv70b, "convert": convert, "decoder": decoder}[args.cmd](args)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -64,9 +64,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
         xp[mt] = reinterpret_cast<const h8_t*>(x) + (long)(xrow[mt] ? m : 0) * kq + j * 4;
     }
 
-    // U K-groups per trip: all loads of the trip are issued before the first MFMA, so one wave keeps
-    // U KiB-sized weight loads (plus their activation fragments) in flight.
-    constexpr int U = (MT == 1) ? 4 : (MT == 2) ? 2 : 1;
+    // U K-groups per trip: all loads of the trip are issued before the first MFMA.  Two is the measured
+    // optimum for narrow waves; deeper batching costs more in occupancy (VGPRs) than it gains.
+    constexpr int U = (MT == 1 && NT <= 2) ? 2 : 1;
     const h8_t ones = {(half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1};
     const h8_t sixteenth = ones * (half_t)0.0625f;
     for (int c0 = wave; c0 < ngroups; c0 += NW * U) {
@@ -213,11 +213,12 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
     return nullptr;
 }
 
-// Default split, from sweeps on MI355X: as many column tiles per wave as still leave roughly 200
-// workgroups (each activation fragment is then reused by more MFMAs), eight waves per workgroup over K.
-static void gemv_default_cfg(int mt, int N, int K, int* nt_out, int* nw_out) {
+// Default split, from sweeps on MI355X.  Eight waves per workgroup over K.  Column tiles per wave: for
+// M <= 8 activation traffic is negligible, so favour occupancy (two tiles); above that reuse each
+// activation fragment for four tiles -- in both cases only while about 200 workgroups remain.
+static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_out) {
     const int strips = (N + 15) / 16, groups = K / 128;
-    int nt = 4;
+    int nt = (M <= 8) ? 2 : 4;
     while (nt > 1 && ((strips + nt - 1) / nt < 192 || gemv_lookup(mt, nt, 8) == nullptr)) nt >>= 1;
     int nw = 8;
     while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
@@ -238,7 +239,7 @@ extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* 
     if (N <= 0 || K <= 0 || (N & 15) || (K & 127))
         return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: need N%%16==0 and K%%128==0, got N=%d K=%d", N, K);
     const int mt = (M + 15) / 16;
-    if (nt <= 0 || nw <= 0) gemv_default_cfg(mt, N, K, &nt, &nw);
+    if (nt <= 0 || nw <= 0) gemv_default_cfg(M, mt, N, K, &nt, &nw);
     gemv_fn fn = gemv_lookup(mt, nt, nw);
     if (!fn) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: no kernel for m-tiles=%d nt=%d nw=%d", mt, nt, nw);
     const int strips = N / 16;
