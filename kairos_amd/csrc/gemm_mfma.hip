@@ -40,6 +40,21 @@ __device__ __forceinline__ void i8x4_to_h2x2(uint32_t w, h2_t& lo, h2_t& hi) {
     hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - k1152;
 }
 
+// One accumulator element, for the epilogues.  The 256 accumulator registers of a 256x256 tile live in
+// AGPRs; left to itself the register allocator copies all of them to VGPRs where the main loop ends and
+// spills over a hundred to scratch.  An explicit read at the point of use keeps each one in place until
+// it is needed.  (The caller leaves >= 18 wait states between the last MFMA and the first read.)
+template <bool FROM_AGPR, typename T>
+__device__ __forceinline__ T acc_elem(T a) {
+    if constexpr (FROM_AGPR) {
+        T v;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+        return v;
+    } else {
+        return a;
+    }
+}
+
 // Split-K: a workgroup that only covers part of K writes its raw accumulators (fp32 or int32, 4 bytes
 // each) to slice `split` of the partial buffer; splitk_reduce_kernel adds the slices in a fixed order
 // and applies the epilogue arithmetic.  Lane layout as in gemm_epilogue below.
@@ -63,7 +78,7 @@ __device__ __forceinline__ void store_partial(const GemmArgs& p, acc_t (&acc)[FM
                     u4_t v;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const auto elem = acc[i][j][4 * g + r];          // copy out of the vector first:
+                        const auto elem = acc_elem<(FM * FN >= 16)>(acc[i][j][4 * g + r]);   // a scalar copy:
                         v[r] = __builtin_bit_cast(uint32_t, elem);       // bit_cast needs an addressable scalar
                     }
                     *reinterpret_cast<u4_t*>(dst + (long)m * N + n) = v;
@@ -152,6 +167,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         }
     } else {
         constexpr int WN = BN / 2;                       // columns per wave
+        constexpr bool BIG = FM * FN >= 16;              // accumulators in AGPRs, read explicitly
         constexpr int PITCH = WN * 2 + 8;                // bytes
         constexpr int CPR = WN * 2 / 16;                 // 16-byte chunks per row
         char* patch = smem + wave * (32 * PITCH);
@@ -189,15 +205,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         float v;
+                        const auto a = acc_elem<BIG>(acc[i][j][4 * g + r]);
                         if constexpr (KIND == KIND_W8A8) {
                             // product rounded to fp32 first, then to fp16 (two roundings, as the
                             // reference epilogue): keep the compiler from fusing them into one
-                            v = (float)acc[i][j][4 * g + r] * ((float)ws4[j][g][r] * as_i[i]);
+                            v = (float)a * ((float)ws4[j][g][r] * as_i[i]);
                             asm volatile("" : "+v"(v));
                         } else if constexpr (KIND == KIND_W8A16) {
-                            v = acc[i][j][4 * g + r] * (float)ws4[j][g][r];
+                            v = a * (float)ws4[j][g][r];
                         } else {
-                            v = acc[i][j][4 * g + r];
+                            v = a;
                         }
                         h[r] = (half_t)v;
                         if constexpr (HAS_BIAS) h[r] = (half_t)((float)h[r] + (float)bs4[j][g][r]);
@@ -227,18 +244,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
     }
 }
 
-// Scheduling hints: spread READS LDS reads, WRITES LDS writes and LOADS global loads evenly between
-// the NMFMA MFMAs of one k-step, so that the matrix pipe never waits behind a burst of memory issue.
+// Scheduling hints: spread WRITES LDS writes evenly between the NMFMA MFMAs of one k-step, READS LDS
+// reads between those of its first half (their results are needed by the next block) and LOADS global
+// loads between those of its second half (a direct-to-LDS load counts as an LDS store, so the compiler
+// keeps it behind every LDS read that precedes it in program order), so that the matrix pipe never
+// waits behind a burst of memory issue.
 template <int NMFMA, int READS, int WRITES, int LOADS, int K = 0>
 __device__ __forceinline__ void sched_interleave() {
     if constexpr (NMFMA >= 4 && K < NMFMA) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        constexpr int r = (K + 1) * READS / NMFMA - K * READS / NMFMA;
+        constexpr int H = NMFMA / 2;                     // LDS reads go behind the first half of the MFMAs
+        constexpr int r = K < H ? (K + 1) * READS / H - K * READS / H : 0;
         constexpr int w = (K + 1) * WRITES / NMFMA - K * WRITES / NMFMA;
-        constexpr int l = (K + 1) * LOADS / NMFMA - K * LOADS / NMFMA;
+        constexpr int l = K >= H ? (K - H + 1) * LOADS / (NMFMA - H) - (K - H) * LOADS / (NMFMA - H) : 0;
         if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
         if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
-        if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x010, l, 0);   // any VMEM: a direct-to-LDS load is not a plain read
         sched_interleave<NMFMA, READS, WRITES, LOADS, K + 1>();
     }
 }
@@ -470,7 +491,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
         mfma_step(1);
     }
 
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();                                         // staging LDS is reused by the epilogue
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");       // MFMA results settle before explicit AGPR reads
     if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
     else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
@@ -612,47 +635,62 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     // A plain barrier instruction (no fence): the fence of __syncthreads would drain every load.
 #define KMI_STAGE_BARRIER(keep) asm volatile("s_waitcnt vmcnt(" #keep ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-    // ---- pipeline: stage t is computed while stages t+1 .. t+NS-1 are in flight.  The MFMAs run one
-    // k-step behind the fragment reads, across the barrier, so LDS latency is never exposed.
+    // ---- pipeline: stage t is computed while stages t+1 .. t+NS-1 are in flight.  Every MFMA block
+    // (one k-step) issues, between its first MFMAs, the fragment reads of the NEXT k-step into the
+    // other register set, so LDS latency hides behind the block and nothing is read after it.
+#define KMI_STAGE_WAIT()                                                   \
+    do {                                                                   \
+        if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);         \
+        else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);      \
+        else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);      \
+        else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);      \
+        else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);      \
+        else KMI_STAGE_BARRIER(0);                                         \
+    } while (0)
+#ifdef KMI_DBG_TIMING
+    const uint64_t dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = wall_clock64();
+#endif
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t) issue_stage(t);
-    static_assert(NS == 4 || NS == 3, "vmcnt immediates below assume 3 or 4 stages");
-    if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);
-    else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);
-    else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);
-    else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);
-    else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);
-    else KMI_STAGE_BARRIER(0);
+    static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
+    KMI_STAGE_WAIT();
     issue_stage(NS - 1);
     read_frags(0, 0, 0);
-    read_frags(0, 1, 1);
-    for (int t = 0; t < T - 1; ++t) {
+    for (int t = 0; t < T; ++t) {
+        read_frags(t, 1, 1);
         mfma_step(0);                                        // (t, step 0)
-        sched_interleave<NMF, 0, 0, 0>();
-        if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);
-        else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);
-        else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);
-        else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);
-        else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);
-        else KMI_STAGE_BARRIER(0);
-        // stage t+1 has landed for every wave; stage t is no longer read by anyone (its fragments
-        // for step 1 sit in registers), so it can take k-stage t+NS
+        sched_interleave<NMF, NRD, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        // stage t+1 has landed for every wave and stage t is fully in registers, so its slot can
+        // take k-stage t+NS
+        KMI_STAGE_WAIT();
+        read_frags(t + 1, 0, 0);                             // past the last stage: a harmless re-read
         issue_stage(t + NS);
-        read_frags(t + 1, 0, 0);
         mfma_step(1);                                        // (t, step 1)
         sched_interleave<NMF, NRD, 0, NLD>();
         __builtin_amdgcn_sched_barrier(0);
-        read_frags(t + 1, 1, 1);
     }
-    mfma_step(0);
-    mfma_step(1);
+#undef KMI_STAGE_WAIT
     // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 #undef KMI_STAGE_BARRIER
+#ifdef KMI_DBG_TIMING
+    const uint64_t dbg_c1 = __builtin_readcyclecounter(), dbg_r1 = wall_clock64();
+#endif
 
     if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
     else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+#ifdef KMI_DBG_TIMING
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (p.splits == 1 && p.partial && tid == 0) {
+        uint64_t* d = static_cast<uint64_t*>(p.partial) + (size_t)blockIdx.x * 8;
+        d[0] = dbg_c0; d[1] = dbg_r0; d[2] = dbg_c1; d[3] = dbg_r1;
+        d[4] = __builtin_readcyclecounter(); d[5] = wall_clock64();
+        uint32_t xcc; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        d[6] = xcc; d[7] = blockIdx.x;
+    }
+#endif
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -712,6 +750,9 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st) {
     const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
     a.splits = pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units);
     a.partial = a.splits > 1 ? g_workspace : nullptr;
+#ifdef KMI_DBG_TIMING
+    a.partial = g_workspace;
+#endif
     const dim3 grid(((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
