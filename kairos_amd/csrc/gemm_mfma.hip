@@ -184,6 +184,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) ws4[j][g] = *reinterpret_cast<const h4_t*>(p.wscales + n);
                 if constexpr (HAS_BIAS) bs4[j][g] = *reinterpret_cast<const h4_t*>(p.bias + n);
             }
+        float wsf[FN][4][4];                              // fp32 once, not once per row block
+        (void)wsf;
+        if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) wsf[j][g][r] = (float)ws4[j][g][r];
+        }
         float as_i[FM];
         (void)as_i;
         if constexpr (KIND == KIND_W8A8) {
@@ -209,10 +219,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                         if constexpr (KIND == KIND_W8A8) {
                             // product rounded to fp32 first, then to fp16 (two roundings, as the
                             // reference epilogue): keep the compiler from fusing them into one
-                            v = (float)a * ((float)ws4[j][g][r] * as_i[i]);
+                            v = (float)a * (wsf[j][g][r] * as_i[i]);
                             asm volatile("" : "+v"(v));
                         } else if constexpr (KIND == KIND_W8A16) {
-                            v = a * (float)ws4[j][g][r];
+                            v = a * wsf[j][g][r];
                         } else {
                             v = a;
                         }
@@ -224,19 +234,28 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 }
             // the patch is private to the wave and LDS serves a wave's requests in order
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            constexpr int NK = 32 * CPR / 64;                // 16-byte chunks per lane and 32-row block
+            u4_t v[NK];
 #pragma unroll
-            for (int k = 0; k < 32 * CPR / 64; ++k) {
-                const int idx = k * 64 + lane, row = idx / CPR, ch = idx % CPR;
-                const u4_t v = *reinterpret_cast<const u4_t*>(patch + row * PITCH + ch * 16);
-                const int m = mw + i * 32 + row, n = nw + ch * 8;
-                if (m < M) {
-                    half_t* dst = outp + (long)m * N + n;
-                    if (wide) {
-                        if (n < N) *reinterpret_cast<u4_t*>(dst) = v;
-                    } else {                             // N % 8 == 4: two 8-byte halves, each whole or absent
-                        if (n < N) *reinterpret_cast<u2_t*>(dst) = u2_t{v[0], v[1]};
-                        if (n + 4 < N) *reinterpret_cast<u2_t*>(dst + 4) = u2_t{v[2], v[3]};
-                    }
+            for (int k = 0; k < NK; ++k) {                   // all reads first: one LDS round trip, not NK
+                const int idx = k * 64 + lane;
+                v[k] = *reinterpret_cast<const u4_t*>(patch + (idx / CPR) * PITCH + (idx % CPR) * 16);
+            }
+            const int n = nw + (lane % CPR) * 8;             // CPR divides 64: the column is the same for every k
+            half_t* dst = outp + (long)(mw + i * 32 + lane / CPR) * N + n;
+            if (wide) {
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
+                    if (m < M && n < N) *reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N) = v[k];
+                }
+            } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
+                    half_t* d = dst + (long)k * (64 / CPR) * N;
+                    if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
+                    if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
@@ -569,9 +588,16 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
         if (16 * (4 * i) < BM) {                             // region lies in the A part (BM % 64 == 0)
             int m = m0 + row;
             m = m < M ? m : M - 1;
+#ifdef KMI_DBG_AROW0
+            m = m0;
+#endif
             voff[i] = (uint32_t)((long)m * row_bytes + c * 16);
         } else if constexpr (TILED_B) {
+#ifdef KMI_DBG_BROW0
+            const int rb = (row - BM) & ~127;
+#else
             const int rb = row - BM;
+#endif
             int strip = rb >> 7;
             if (n0 + strip * KMI_TILE_N >= N) strip = 0;
             voff[i] = (uint32_t)((long)strip * T_all * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
@@ -581,13 +607,16 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
             voff[i] = (uint32_t)((long)n * row_bytes + c * 16);
         }
     }
-    auto issue_stage = [&](int t) {                          // k-stage t -> LDS stage t % NS
+    // k-stage t -> LDS stage t % NS; the loads of a stage are issued in two halves (h = 0, 1)
+    constexpr int NLD0 = (NLD + 1) / 2;
+    auto issue_half = [&](int t, int h) {
         const int tt = t0 + (t < T ? t : T - 1);             // past the end: harmless reload into a free stage
         char* dst = smem + (t % NS) * STAGE + wave * 1024;
         const char* ab = a_base + (long)tt * 64;
         const char* bb = b_base + (long)tt * B_STEP;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
+            if ((i < NLD0) != (h == 0)) continue;
 #ifdef KMI_DBG_NOLOAD
             if (t >= NS) continue;
 #endif
@@ -595,6 +624,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
             __builtin_amdgcn_global_load_lds((global_void_ptr)g, (lds_void_ptr)(dst + i * 4096), 16, 0, 0);
         }
     };
+    auto issue_stage = [&](int t) { issue_half(t, 0); issue_half(t, 1); };
 
     // ---- fragment addressing: lane (r = lane&31, kh = lane>>5) reads chunk 2s+kh of row base+r
     const int fr = lane & 31, fkh = lane >> 5;
@@ -633,7 +663,11 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
 
     // Wait until at most `keep` direct loads of this thread are outstanding, then meet the other waves.
     // A plain barrier instruction (no fence): the fence of __syncthreads would drain every load.
+#ifdef KMI_DBG_NOWAIT
+#define KMI_STAGE_BARRIER(keep) asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#else
 #define KMI_STAGE_BARRIER(keep) asm volatile("s_waitcnt vmcnt(" #keep ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#endif
 
     // ---- pipeline: stage t is computed while stages t+1 .. t+NS-1 are in flight.  Every MFMA block
     // (one k-step) issues, between its first MFMAs, the fragment reads of the NEXT k-step into the
@@ -654,20 +688,23 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     for (int t = 0; t < NS - 1; ++t) issue_stage(t);
     static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
     KMI_STAGE_WAIT();
-    issue_stage(NS - 1);
+    issue_half(NS - 1, 0);
     read_frags(0, 0, 0);
     for (int t = 0; t < T; ++t) {
+        // Slot (t-1) % NS was released by the previous barrier: it takes k-stage t+NS-1, half of the
+        // loads in each of the two MFMA blocks that follow that barrier, so the memory pipe sees one
+        // load per wave every few MFMAs instead of a burst.
         read_frags(t, 1, 1);
+        issue_half(t + NS - 1, 1);
         mfma_step(0);                                        // (t, step 0)
-        sched_interleave<NMF, NRD, 0, 0>();
+        sched_interleave<NMF, NRD, 0, NLD - NLD0>();
         __builtin_amdgcn_sched_barrier(0);
-        // stage t+1 has landed for every wave and stage t is fully in registers, so its slot can
-        // take k-stage t+NS
+        // stage t+1 has landed for every wave and stage t is fully in registers
         KMI_STAGE_WAIT();
         read_frags(t + 1, 0, 0);                             // past the last stage: a harmless re-read
-        issue_stage(t + NS);
+        issue_half(t + NS, 0);
         mfma_step(1);                                        // (t, step 1)
-        sched_interleave<NMF, NRD, 0, NLD>();
+        sched_interleave<NMF, NRD, 0, NLD0>();
         __builtin_amdgcn_sched_barrier(0);
     }
 #undef KMI_STAGE_WAIT
