@@ -538,6 +538,7 @@ typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
 template <int KIND, int BM, int BN, bool TILED_B, int NS>
 __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass cannot instantiate code that uses the buffer resource type
     constexpr bool I8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     static_assert(KIND == KIND_F16 || I8, "direct staging copies operands verbatim");
     constexpr int FM = BM / 64, FN = BN / 64;
@@ -609,19 +610,25 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     }
     // k-stage t -> LDS stage t % NS; the loads of a stage are issued in two halves (h = 0, 1)
     constexpr int NLD0 = (NLD + 1) / 2;
+    // Buffer addressing: a resource per operand (base pointer, no stride, no range limit), the per-lane
+    // 32-bit offset that never changes and a scalar offset that advances with the k-stage, so a load
+    // reads one address VGPR per lane and the loop carries no vector address arithmetic at all.
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a_base), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b_base), 0, -1, 0x00020000);
     auto issue_half = [&](int t, int h) {
         const int tt = t0 + (t < T ? t : T - 1);             // past the end: harmless reload into a free stage
         char* dst = smem + (t % NS) * STAGE + wave * 1024;
-        const char* ab = a_base + (long)tt * 64;
-        const char* bb = b_base + (long)tt * B_STEP;
+        const uint32_t sa = (uint32_t)tt * 64u, sb = (uint32_t)tt * (uint32_t)B_STEP;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             if ((i < NLD0) != (h == 0)) continue;
 #ifdef KMI_DBG_NOLOAD
             if (t >= NS) continue;
 #endif
-            const char* g = ((16 * (4 * i) < BM) ? ab : bb) + voff[i];
-            __builtin_amdgcn_global_load_lds((global_void_ptr)g, (lds_void_ptr)(dst + i * 4096), 16, 0, 0);
+            if (16 * (4 * i) < BM)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, voff[i], sa, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_ptr)(dst + i * 4096), 16, voff[i], sb, 0, 0);
         }
     };
     auto issue_stage = [&](int t) { issue_half(t, 0); issue_half(t, 1); };
@@ -727,6 +734,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
         uint32_t xcc; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
         d[6] = xcc; d[7] = blockIdx.x;
     }
+#endif
 #endif
 }
 
