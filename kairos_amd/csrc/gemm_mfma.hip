@@ -247,7 +247,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
 #pragma unroll
                 for (int k = 0; k < NK; ++k) {
                     const int m = mw + i * 32 + (k * 64 + lane) / CPR;
-                    if (m < M && n < N) *reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N) = v[k];
+                    if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N));
                 }
             } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
 #pragma unroll
