@@ -374,41 +374,50 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     if constexpr (KIND == KIND_W8A16) b_step = 64;
     else b_step = 128;
 
-    u4_t ra[A_CH];
-    u4_t rb[B_CH];
-    half_t rs[B_CH], rz[B_CH];
+    // Two register sets hold k-tiles in flight between global memory and LDS: tile t travels in set
+    // t & 1, is loaded about two iterations before it is written to LDS, and the set index is a
+    // compile-time constant everywhere (the main loop is unrolled by two), so the compiler can count
+    // exactly how many newer loads may stay outstanding at each use.
+    u4_t ra[2][A_CH];
+    u4_t rb[2][B_CH];
+    half_t rs[2][B_CH], rz[2][B_CH];
     (void)rs; (void)rz;
+    using set0 = std::integral_constant<int, 0>;
+    using set1 = std::integral_constant<int, 1>;
 
-    auto load_tile = [&](int kt) {
+    auto load_tile = [&](auto set, int kt_req) {
+        constexpr int S = decltype(set)::value;
+        const int kt = kt_req < KT ? kt_req : KT - 1;        // past the end: a harmless reload, never stored
 #pragma unroll
-        for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u4_t*>(pa[i] + (long)(kt0 + kt) * 128);
+        for (int i = 0; i < A_CH; ++i) ra[S][i] = *reinterpret_cast<const u4_t*>(pa[i] + (long)(kt0 + kt) * 128);
 #pragma unroll
         for (int i = 0; i < B_CH; ++i) {
-            rb[i] = *reinterpret_cast<const u4_t*>(pb[i] + (long)(kt0 + kt) * b_step);
+            rb[S][i] = *reinterpret_cast<const u4_t*>(pb[i] + (long)(kt0 + kt) * b_step);
             if constexpr (KIND == KIND_W4A16) {
-                rs[i] = p.scales[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
-                rz[i] = p.szeros[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
+                rs[S][i] = p.scales[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
+                rz[S][i] = p.szeros[(long)((kt0 + kt) >> 1) * N + scale_col[i]];
             }
         }
     };
 
-    auto store_tile = [&](int stage) {
+    auto store_tile = [&](auto set, int stage) {
+        constexpr int S = decltype(set)::value;
         char* sa = smem + stage * STAGE;
         char* sb = sa + BM * 128;
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
             const int q = tid + i * 256;
-            *reinterpret_cast<u4_t*>(sa + lds_off(q >> 3, q & 7)) = ra[i];
+            *reinterpret_cast<u4_t*>(sa + lds_off(q >> 3, q & 7)) = ra[S][i];
         }
         if constexpr (KIND == KIND_W4A16) {
 #pragma unroll
             for (int i = 0; i < B_CH; ++i) {
                 const int q = tid + i * 256, row = q >> 1, h = q & 1;
-                const h2_t s2 = {rs[i], rs[i]}, z2 = {rz[i], rz[i]};
-                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 0)) = dequant_nibble<0>(rb[i], s2, z2);
-                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 1)) = dequant_nibble<1>(rb[i], s2, z2);
-                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 2)) = dequant_nibble<2>(rb[i], s2, z2);
-                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 3)) = dequant_nibble<3>(rb[i], s2, z2);
+                const h2_t s2 = {rs[S][i], rs[S][i]}, z2 = {rz[S][i], rz[S][i]};
+                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 0)) = dequant_nibble<0>(rb[S][i], s2, z2);
+                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 1)) = dequant_nibble<1>(rb[S][i], s2, z2);
+                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 2)) = dequant_nibble<2>(rb[S][i], s2, z2);
+                *reinterpret_cast<h8_t*>(sb + lds_off(row, 4 * h + 3)) = dequant_nibble<3>(rb[S][i], s2, z2);
             }
         } else if constexpr (KIND == KIND_W8A16) {
 #pragma unroll
@@ -416,7 +425,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
                 const int q = tid + i * 256, row = q >> 2, c = q & 3;
                 h2_t v[8];
 #pragma unroll
-                for (int w = 0; w < 4; ++w) i8x4_to_h2x2(rb[i][w], v[2 * w], v[2 * w + 1]);
+                for (int w = 0; w < 4; ++w) i8x4_to_h2x2(rb[S][i][w], v[2 * w], v[2 * w + 1]);
                 h8_t lo, hi;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -430,7 +439,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
             for (int i = 0; i < B_CH; ++i) {
                 const int q = tid + i * 256;
-                *reinterpret_cast<u4_t*>(sb + lds_off(q >> 3, q & 7)) = rb[i];
+                *reinterpret_cast<u4_t*>(sb + lds_off(q >> 3, q & 7)) = rb[S][i];
             }
         }
     };
@@ -462,17 +471,25 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     constexpr bool PURE_COPY = (KIND == KIND_F16 || I8);     // staging without conversion ALU work
     constexpr int NMF = FM * FN, NRD = FM + FN, NWR = PURE_COPY ? A_CH + B_CH : 0, NLD = A_CH + B_CH;
 
-    // ---- software pipeline.  LDS stage t&1 holds k-tile t.  Per k-tile:
+    // ---- software pipeline.  LDS stage t&1 holds k-tile t.  Per k-tile kt:
     //   steps 0,1: MFMAs + fragment reads of the next step
-    //   step 2   : MFMAs + fragment reads of step 3 + write k-tile t+1 (already in registers) to the other stage
+    //   step 2   : MFMAs + fragment reads of step 3 + write k-tile kt+1 (in registers since iteration kt-2)
+    //              to the other stage
     //   barrier  : the other stage is complete, this stage is no longer read
-    //   step 3   : MFMAs + fragment reads of step 0 of k-tile t+1 + global loads of k-tile t+2
-    load_tile(0);
-    store_tile(0);
-    if (KT > 1) load_tile(1);
+    //   step 3   : MFMAs + fragment reads of step 0 of k-tile kt+1 + global loads of k-tile kt+3 into the
+    //              register set just emptied
+    load_tile(set0{}, 0);
+    store_tile(set0{}, 0);
+    // the loads of the two tiles must be issued in the loop's own order (all of k-tile 1, then all of
+    // k-tile 2): the wait counts inside the loop are the merge of this state and the back edge's
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile(set1{}, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile(set0{}, 2);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     read_frags(0, 0, 0);
-    for (int kt = 0; kt < KT - 1; ++kt) {
+    auto body = [&](auto set, int kt) {                       // `set` holds k-tile kt+1
         const int cur = kt & 1, nxt = cur ^ 1;
         read_frags(cur, 1, 1);
         mfma_step(0);
@@ -483,16 +500,22 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
         sched_interleave<NMF, NRD, 0, 0>();
         __builtin_amdgcn_sched_barrier(0);
         read_frags(cur, 3, 1);
-        store_tile(nxt);
+        store_tile(set, nxt);
         mfma_step(0);
         sched_interleave<NMF, NRD, NWR, 0>();
         __syncthreads();
         read_frags(nxt, 0, 0);
-        if (kt + 2 < KT) load_tile(kt + 2);
+        load_tile(set, kt + 3);
         mfma_step(1);
         sched_interleave<NMF, NRD, 0, NLD>();
         __builtin_amdgcn_sched_barrier(0);
+    };
+    int kt = 0;
+    for (; kt + 2 <= KT - 1; kt += 2) {
+        body(set1{}, kt);
+        body(set0{}, kt + 1);
     }
+    if (kt < KT - 1) body(set1{}, kt);
     {   // last k-tile: nothing left to stage
         const int cur = (KT - 1) & 1;
         read_frags(cur, 1, 1);
