@@ -775,17 +775,21 @@ extern "C" int kmi_gemm_set_workspace(void* ptr, size_t bytes) {
 static thread_local int g_force_splits = 0;
 extern "C" void kmi_gemm_force_splits(int splits) { g_force_splits = splits; }
 
-// Number of K splits: only when the output tiles alone cannot occupy the chip, every split keeps at
-// least four 128-byte k-tiles, and the partial sums fit the registered workspace.
+// Number of K splits: only while the split workgroups still fit one round over the 256 CUs (a second
+// round costs more than the idle CUs of the first), every split keeps at least eight 128-byte k-tiles,
+// and the partial sums fit the registered workspace.  Measured on MI355X: splitting 192 or 224 tiles in
+// two is 1.3-2x slower than running them as they are.
 static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
     const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     int s = 1;
-    if (g_force_splits > 0) s = g_force_splits;
-    else if (tiles < 256) {
-        s = (int)(512 / tiles);
+    if (g_force_splits > 0) {
+        s = g_force_splits;
+        if (s > ktiles / 4) s = ktiles / 4;
+    } else {
+        s = (int)(256 / tiles);
         if (s > 8) s = 8;
+        if (s > ktiles / 8) s = ktiles / 8;
     }
-    if (s > ktiles / 4) s = ktiles / 4;
     const size_t per = (size_t)M * N * 4;
     if (per == 0 || g_workspace == nullptr) return 1;
     if ((size_t)s * per > g_workspace_bytes) s = (int)(g_workspace_bytes / per);
@@ -833,7 +837,7 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st) {
 // Tile choice: the largest tile that still yields about one workgroup per CU.
 static int pick_tile(int M, int N) {
     auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M > 128 && wgs(256, 256) >= 200) return 256;
+    if (M > 128 && wgs(256, 256) >= 180) return 256;
     if (M > 64 && wgs(128, 128) >= 128) return 128;
     return 64;
 }
