@@ -80,20 +80,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 u[t][nt] = __builtin_nontemporal_load(wp[nt] + c * 16);
-#ifdef KMI_DBG_NOSCALE
-                s[t][nt] = (half_t)1.0f; z[t][nt] = (half_t)0.5f;
-#else
                 s[t][nt] = scales[(long)c * N + ncol[nt]];
                 z[t][nt] = szeros[(long)c * N + ncol[nt]];
-#endif
             }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-#ifdef KMI_DBG_NOX
-                if (false) {
-#else
                 if (xrow[mt]) {
-#endif
 #pragma unroll
                     for (int a = 0; a < 4; ++a) xa[t][mt][a] = xp[mt][c * 16 + a];
                 } else {
