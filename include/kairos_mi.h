@@ -77,6 +77,14 @@ int kmi_untile(void* out_rowmajor, const void* tiled, int N, int K, int elem_siz
  * kernels/csrc/kairos_kernel/quant/quant_f16_to_i8.cu:86-104).  Needs K%8==0, K<=32768. */
 int kmi_quant_act_i8(void* out_i8, void* scale_f16, const void* x_f16, int M, int K, void* stream);
 
+/* Both preparation steps of the W8A8 lane in ONE launch: kmi_cvt_i4_to_i8 (tiled != 0: kmi_cvt_i4_to_i8_tiled)
+ * into w8_out and kmi_quant_act_i8 of x into a8_out / ascale_f16.  The results are bit-identical to the two
+ * separate calls; the shared launch saves a kernel boundary on every call that has to convert.  No reference
+ * counterpart (the reference issues the two kernels one after the other, kairos/dynamic_linear.py:150-162).
+ * Argument rules as for the two separate entry points. */
+int kmi_prep_w8a8(void* w8_out, int tiled, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
+                  int N, int K, int G, void* a8_out, void* ascale_f16, const void* x_f16, int M, void* stream);
+
 /* ---- W4A16, small M ---------------------------------------------------------------------------- */
 
 /* out = x . dequant(qweight)^T (+bias), weights streamed once, fp32 accumulation on MFMA.

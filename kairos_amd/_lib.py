@@ -22,6 +22,7 @@ SIGNATURES = {
     "kmi_cvt_i4_to_i8_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_untile": [_P, _P, _I, _I, _I, _P],
     "kmi_quant_act_i8": [_P, _P, _P, _I, _I, _P],
+    "kmi_prep_w8a8": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P, _I, _P],
     "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

@@ -2,90 +2,14 @@
 // the tiled layout the MFMA GEMMs copy straight into LDS.  Pure streaming kernels: every thread
 // reads one 16-byte chunk (32 weights of one row, K-contiguous after decoding) and writes 64 or 32
 // contiguous bytes.  Bound by HBM bandwidth: N*K/2 bytes in, N*K*{2,1} bytes out.
-#include "kmi_common.h"
-
-enum { OUT_F16 = 0, OUT_I8 = 1, OUT_F16_TILED = 2, OUT_I8_TILED = 3 };
-
-__device__ __forceinline__ uint32_t pack_i8x4(h2_t a, h2_t b) {
-    // truncate toward zero after clipping to the int8 range (clip first: the cast is then exact)
-    const h2_t lo = {(half_t)-128.0f, (half_t)-128.0f};
-    const h2_t hi = {(half_t)127.0f, (half_t)127.0f};
-    a = __builtin_elementwise_min(__builtin_elementwise_max(a, lo), hi);
-    b = __builtin_elementwise_min(__builtin_elementwise_max(b, lo), hi);
-    const uint32_t b0 = (uint32_t)(uint8_t)(int8_t)(short)a[0];
-    const uint32_t b1 = (uint32_t)(uint8_t)(int8_t)(short)a[1];
-    const uint32_t b2 = (uint32_t)(uint8_t)(int8_t)(short)b[0];
-    const uint32_t b3 = (uint32_t)(uint8_t)(int8_t)(short)b[1];
-    return b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-}
-
-__device__ __forceinline__ u2_t h8_to_i8x8(h8_t v) {
-    h2_t p0 = {v[0], v[1]}, p1 = {v[2], v[3]}, p2 = {v[4], v[5]}, p3 = {v[6], v[7]};
-    u2_t o;
-    o[0] = pack_i8x4(p0, p1);
-    o[1] = pack_i8x4(p2, p3);
-    return o;
-}
+#include "prep_bodies.h"
 
 template <int OUT>
 __global__ __launch_bounds__(256) void cvt_i4_kernel(void* __restrict__ out, const u4_t* __restrict__ qw,
                                                      const half_t* __restrict__ scales,
                                                      const half_t* __restrict__ szeros, int N, int K,
                                                      long total_chunks) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total_chunks) return;
-    const int per_quad = K >> 3;                 // 16-byte chunks per four-row block
-    const int quad = (int)(i / per_quad);
-    const int rem = (int)(i - (long)quad * per_quad);
-    const int kb64 = rem >> 3;
-    const int r = (rem >> 1) & 3;
-    const int h = rem & 1;
-    const int n = quad * 4 + r;
-    const int k0 = kb64 * 64 + h * 32;
-    const int g = k0 >> 7;
-
-    const u4_t u = __builtin_nontemporal_load(qw + i);
-    const half_t s = scales[(long)g * N + n];
-    const half_t z = szeros[(long)g * N + n];
-    const h2_t s2 = {s, s};
-    const h2_t z2 = {z, z};
-    const h8_t w0 = dequant_nibble<0>(u, s2, z2);
-    const h8_t w1 = dequant_nibble<1>(u, s2, z2);
-    const h8_t w2 = dequant_nibble<2>(u, s2, z2);
-    const h8_t w3 = dequant_nibble<3>(u, s2, z2);
-
-    if constexpr (OUT == OUT_F16) {
-        h8_t* o = reinterpret_cast<h8_t*>(reinterpret_cast<half_t*>(out) + (long)n * K + k0);
-        o[0] = w0; o[1] = w1; o[2] = w2; o[3] = w3;
-    } else if constexpr (OUT == OUT_I8) {
-        u4_t* o = reinterpret_cast<u4_t*>(reinterpret_cast<int8_t*>(out) + (long)n * K + k0);
-        const u2_t a = h8_to_i8x8(w0), b = h8_to_i8x8(w1), c = h8_to_i8x8(w2), d = h8_to_i8x8(w3);
-        u4_t lo = {a[0], a[1], b[0], b[1]};
-        u4_t hi = {c[0], c[1], d[0], d[1]};
-        o[0] = lo; o[1] = hi;
-    } else if constexpr (OUT == OUT_F16_TILED) {
-        // tile = 128 rows x 32 fp16 (8 KiB): this thread's 32 weights are exactly one tile row;
-        // chunk c of row r sits at c ^ ((r>>2)&3)
-        const int row = n & (KMI_TILE_N - 1);
-        const long tile = (long)(n / KMI_TILE_N) * (K >> 5) + (kb64 * 2 + h);
-        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 64) + row * 64;
-        const int sw = (row >> 2) & 3;
-        *reinterpret_cast<h8_t*>(base + ((0 ^ sw) << 4)) = w0;
-        *reinterpret_cast<h8_t*>(base + ((1 ^ sw) << 4)) = w1;
-        *reinterpret_cast<h8_t*>(base + ((2 ^ sw) << 4)) = w2;
-        *reinterpret_cast<h8_t*>(base + ((3 ^ sw) << 4)) = w3;
-    } else {
-        // tile = 128 rows x 64 int8 (8 KiB): this thread's 32 weights are half of one tile row
-        const int row = n & (KMI_TILE_N - 1);
-        const long tile = (long)(n / KMI_TILE_N) * (K >> 6) + kb64;
-        char* base = reinterpret_cast<char*>(out) + tile * (KMI_TILE_N * 64) + row * 64;
-        const int sw = (row >> 2) & 3;
-        const u2_t a = h8_to_i8x8(w0), b = h8_to_i8x8(w1), c = h8_to_i8x8(w2), d = h8_to_i8x8(w3);
-        u4_t lo = {a[0], a[1], b[0], b[1]};
-        u4_t hi = {c[0], c[1], d[0], d[1]};
-        *reinterpret_cast<u4_t*>(base + (((2 * h + 0) ^ sw) << 4)) = lo;
-        *reinterpret_cast<u4_t*>(base + (((2 * h + 1) ^ sw) << 4)) = hi;
-    }
+    cvt_i4_body<OUT>((long)blockIdx.x * 256 + threadIdx.x, out, qw, scales, szeros, N, K, total_chunks);
 }
 
 // tiled -> row-major (verification helper): one thread per 16-byte chunk

@@ -137,10 +137,15 @@ class DynamicLinear(torch.nn.Module):
         elif comp_type in (_W4A16_GEMM, _W4A16_GEMV):
             out = ops.gemm_forward(x, self.qweight, self.scales, self.scaled_zeros, bias=self.bias)
         elif comp_type == _W8A8:
-            w8, tiled = self._converted('i8')
             int_x = torch.empty_like(x, dtype=torch.int8)
             scale_x = torch.empty((m,), device=x.device, dtype=torch.float16)
-            ops.quant_fp16_to_int8(int_x, x, scale_x)
+            tiled = self._tileable()
+            w8, hit = self._cache().get(self._uid, ('i8', tiled), self.shape, torch.int8, self.qweight.device)
+            if hit:
+                ops.quant_fp16_to_int8(int_x, x, scale_x)
+            else:                                            # conversion and quantisation share one launch
+                ops.prep_w8a8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8, int_x, x, scale_x,
+                              self.group_size, tiled=tiled)
             out = torch.empty((m, N), device=x.device, dtype=torch.float16)
             ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
         elif comp_type in (_W8A16_GEMM, _W8A16_GEMV):

@@ -95,6 +95,21 @@ def quant_fp16_to_int8(out, input, scale):
           M, K, _stream())
 
 
+def prep_w8a8(w8_out, qweight, scale_to8, scaled_zero_to8, int_x, x, scale_x, group_size=GROUP_SIZE, tiled=False):
+    """int4 -> int8 weight conversion and per-token activation quantisation in one launch (bit-identical to
+    dequant_interleaved_int4_to_int8 followed by quant_fp16_to_int8)."""
+    _need(w8_out, torch.int8, "w8_out"); _need(qweight, torch.int16, "qweight")
+    _need(scale_to8, torch.float16, "scale_to8"); _need(scaled_zero_to8, torch.float16, "scaled_zero_to8")
+    _need(int_x, torch.int8, "int_x"); _need(x, torch.float16, "x"); _need(scale_x, torch.float16, "scale_x")
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    if x.shape[-1] != K:
+        raise ValueError(f"prep_w8a8: x has {x.shape[-1]} columns, the weight {K}")
+    M = x.numel() // K
+    _call("prep_w8a8", M, N, K, _lib.load().kmi_prep_w8a8, w8_out.data_ptr(), 1 if tiled else 0, qweight.data_ptr(),
+          scale_to8.data_ptr(), scaled_zero_to8.data_ptr(), N, K, group_size, int_x.data_ptr(), scale_x.data_ptr(),
+          x.data_ptr(), M, _stream())
+
+
 # ---- products -----------------------------------------------------------------------------------
 def _flat2d(x):
     return x.reshape(-1, x.shape[-1])

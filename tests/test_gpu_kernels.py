@@ -337,3 +337,34 @@ def test_argument_errors(ops):
     assert e.value.code == -4
     with pytest.raises(TypeError):
         ops.quant_fp16_to_int8(torch.empty((4, K), dtype=torch.int8, device="cuda"), x.float(), torch.empty(4, dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (7, 256, 512), (300, 384, 1024), (64, 128, 4096)])
+def test_prep_w8a8_equals_separate_kernels(ops, tiled, M, N, K):
+    """The fused launch (conversion + activation quantiser) gives the bits of the two stand-alone entry points."""
+    import torch
+    w = O.synth_weights(N, K, N + K)
+    pw = O.prepare_weights(w, 128)
+    dev = "cuda"
+    qw = torch.from_numpy(pw["qweight"]).to(dev)
+    s8 = torch.from_numpy(pw["scales_to8"]).to(dev)
+    z8 = torch.from_numpy(pw["scaled_zeros_to8"]).to(dev)
+    x = torch.from_numpy(O.synth_acts(M, K, M)).to(dev)
+    x[0, :] = 0 if M > 3 else x[0, :]                       # an all-zero token among the rows
+    w_ref = torch.empty((N, K), dtype=torch.int8, device=dev)
+    ops.dequant_interleaved_int4_to_int8(w_ref, qw, s8, z8, 128, tiled=tiled)
+    a_ref = torch.empty((M, K), dtype=torch.int8, device=dev)
+    sc_ref = torch.empty((M,), dtype=torch.float16, device=dev)
+    ops.quant_fp16_to_int8(a_ref, x, sc_ref)
+    w_f = torch.full((N, K), 77, dtype=torch.int8, device=dev)
+    a_f = torch.full((M, K), 77, dtype=torch.int8, device=dev)
+    sc_f = torch.full((M,), 3.0, dtype=torch.float16, device=dev)
+    ops.prep_w8a8(w_f, qw, s8, z8, a_f, x, sc_f, 128, tiled=tiled)
+    assert torch.equal(w_f, w_ref)
+    assert torch.equal(a_f, a_ref)
+    assert torch.equal(sc_f.view(torch.int16), sc_ref.view(torch.int16))
+    # and against the oracle directly
+    a_o, sc_o = O.quant_act_i8(x.cpu().numpy())
+    assert np.array_equal(a_f.cpu().numpy(), a_o)
