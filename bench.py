@@ -148,6 +148,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="layer copies rotated to defeat the Infinity Cache")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-lane sweep table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--lut", default=None, help="directory holding seg_perf_list.pt (default: the committed MI355X table)")
     ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -198,7 +199,10 @@ def main():
     shapes = [(N, K) for _, N, K in LAYER]
     prof = Profiler(shapes)
     lut_source = "committed MI355X table"
-    if os.path.exists(os.path.join(LUT_DIR, "seg_perf_list.pt")):
+    if args.lut:
+        prof.load(args.lut.rstrip("/") + "/")
+        lut_source = "table given by --lut"
+    elif os.path.exists(os.path.join(LUT_DIR, "seg_perf_list.pt")):
         prof.load(LUT_DIR + "/")
     else:
         lut_source = "profiled at start-up (n=20)"
