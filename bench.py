@@ -148,6 +148,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="layer copies rotated to defeat the Infinity Cache")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-lane sweep table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the small-M layers")
     ap.add_argument("--lut", default=None, help="directory holding seg_perf_list.pt (default: the committed MI355X table)")
     ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -283,6 +284,25 @@ def main():
                 layers[li][i % args.copies](acts[(M, K)])
         by_m[M] = round(time_calls(layer_call, n), 2)
 
+    # ---- the same layers replayed from a HIP graph (one graph per M: all layer copies, four linears each):
+    # what the kernels cost once the ~9 us of host work per call is out of the way.  Reported beside the
+    # eager figures, never instead of them.
+    graph_by_m = {}
+    if not args.no_graph:
+        from kairos_amd.graphed import GraphedCallable
+        for M in [m for m in M_GRID if m <= 256]:
+            xs = [acts[(M, K)] for (_n, _N, K) in LAYER]
+
+            def graph_step(*inputs, M=M):
+                outs = []
+                for c in range(args.copies):
+                    for li in range(len(LAYER)):
+                        outs.append(layers[li][c](inputs[li]))
+                return tuple(outs)
+            g = GraphedCallable(graph_step, xs)
+            graph_by_m[M] = round(time_calls(lambda i=0: g.replay(), 20) / args.copies, 2)
+            del g
+
     sweep = []
     if not args.no_sweep:
         lanes = ["w4a16_gemv", "w4a16_gemm", "w8a16_gemm", "w8a8", "fp16"]
@@ -349,6 +369,7 @@ def main():
         "wall_s_timed_region": round(wall, 3),
         "conversion_share_of_kernel_time": round(conv_sec / total_kernel_sec, 4),
         "kernels": kernels, "us_per_layer_by_m": by_m,
+        "graph_replay_us_per_layer_by_m": graph_by_m,
         "best_small_m": small and {k: small[k] for k in ("shape", "M", "us", "gbps", "roofline_frac")},
         "best_large_m": large and {k: large[k] for k in ("shape", "M", "lane", "us", "tflops", "roofline_frac")},
         "config1_gemv_us": round(cfg1_us, 2),

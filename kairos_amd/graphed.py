@@ -1,0 +1,90 @@
+"""HIP-graph replay of a fixed sequence of switched linears.
+
+Decode-sized calls are bound by the host (about 9 us of Python, allocation and launch per linear against
+4-15 us of kernel time), not by the kernels.  A caller whose step has fixed shapes -- one decode step at a
+given batch size -- can capture it once and replay it with a single graph launch.  The lookup table is
+consulted while capturing, so a graph is tied to the M it was captured with: capture one per batch bucket,
+exactly as serving stacks do with CUDA graphs.
+
+Capture rules this module enforces or relies on:
+  * every kernel of the library launches on torch's current stream, so torch's stream capture records it;
+  * the library records no memset nodes (none of its entry points clears memory);
+  * the temp cache and the split-K workspace are created BEFORE capture (they must not be allocated from
+    the graph's private pool, other graphs and eager calls share them);
+  * the temp cache is invalidated right before capture, so every conversion the step needs is part of the
+    graph, and after every replay, because the graph rewrites the cache behind the host-side tag's back;
+  * inputs are copied into static buffers before each replay; outputs are the static tensors captured.
+"""
+import torch
+
+from . import ops
+from .temp_cache import default_cache
+
+
+class GraphedCallable:
+    """Captures `fn(*static_inputs)` once; `__call__(*inputs)` copies the inputs in and replays.
+
+    `fn` must be a pure function of its tensor arguments over modules of this package (fixed shapes, no
+    host-side data dependence).  The returned tensors are reused by every replay: consume or clone them
+    before the next call.
+    """
+
+    def __init__(self, fn, example_inputs, warmup=3, caches=None):
+        """caches: the TempCache objects the captured modules use (default: the process-wide one)."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("GraphedCallable: needs a GPU")
+        self._static_in = [x.clone() for x in example_inputs]
+        ops.ensure_workspace(device=self._static_in[0].device)
+        side = torch.cuda.Stream()                      # default priority
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):                     # sizes the temp cache, settles the LUT memo
+                fn(*self._static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self._caches = list(caches) if caches is not None else [default_cache()]
+        self._invalidate()
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._static_out = fn(*self._static_in)
+        self._invalidate()
+        self.replays = 0
+
+    def _invalidate(self):
+        for c in self._caches:
+            c.invalidate()
+
+    def __call__(self, *inputs):
+        if len(inputs) != len(self._static_in):
+            raise ValueError(f"GraphedCallable: captured with {len(self._static_in)} inputs, got {len(inputs)}")
+        for dst, src in zip(self._static_in, inputs):
+            if dst.shape != src.shape or dst.dtype != src.dtype:
+                raise ValueError(f"GraphedCallable: captured for {tuple(dst.shape)} {dst.dtype}, "
+                                 f"got {tuple(src.shape)} {src.dtype}")
+            if dst.data_ptr() != src.data_ptr():
+                dst.copy_(src)
+        self._graph.replay()
+        self._invalidate()
+        self.replays += 1
+        return self._static_out
+
+    def replay(self):
+        """Replays on the inputs already in the static buffers (no copies)."""
+        self._graph.replay()
+        self._invalidate()
+        self.replays += 1
+        return self._static_out
+
+    @property
+    def static_inputs(self):
+        return self._static_in
+
+
+def graph_layer(linears, example_input_for):
+    """Convenience: one graph over `[lin(x) for lin in linears]`, `example_input_for(lin)` giving each input."""
+    xs = [example_input_for(l) for l in linears]
+
+    def step(*inputs):
+        return tuple(l(x) for l, x in zip(linears, inputs))
+
+    return GraphedCallable(step, xs)

@@ -123,3 +123,41 @@ def test_profiler_builds_a_table(gpu, tmp_path):
         assert again.get_comp_type((256, 512), m) == prof.get_comp_type((256, 512), m)
     text = open(tmp_path / "seg_perf_list.pt").read()
     assert json.loads(text) == prof.seg_perf_list
+
+
+@pytest.mark.gpu
+def test_graph_replay_matches_eager():
+    """A captured layer step replays to the eager bits, several times, with eager work between the replays."""
+    import torch
+    from kairos_amd.dynamic_linear import DynamicLinear
+    from kairos_amd.graphed import GraphedCallable
+
+    class FixedLut:                      # small-M lane for the first linear, W8A8 (conversion in the graph) for the second
+        def __init__(self): self.table = {}
+        def get_comp_type(self, shape, m): return self.table[shape]
+
+    torch.manual_seed(3)
+    l1 = DynamicLinear.from_module(torch.nn.Linear(512, 256, bias=True, dtype=torch.float16), device="cuda")
+    l2 = DynamicLinear.from_module(torch.nn.Linear(256, 384, bias=False, dtype=torch.float16), device="cuda")
+    l3 = DynamicLinear.from_module(torch.nn.Linear(512, 128, bias=False, dtype=torch.float16), device="cuda")
+    lut = FixedLut()
+    lut.table = {(256, 512): 1, (384, 256): 2, (128, 512): 2}
+    old = DynamicLinear.prof
+    DynamicLinear.prof = lut
+    try:
+        def step(x):
+            return l2(l1(x)), l3(x)
+        xs = [torch.randn(1, 8, 512, device="cuda", dtype=torch.float16) for _ in range(4)]
+        eager = [tuple(t.clone() for t in step(x)) for x in xs]
+        g = GraphedCallable(step, [xs[0]])
+        for rep in range(3):
+            for x, want in zip(xs, eager):
+                got = g(x)
+                assert all(torch.equal(a, b) for a, b in zip(got, want)), f"replay {rep}"
+                # eager work on another layer in between: it overwrites the shared temp cache
+                again = step(xs[(rep + 1) % 4])
+                assert all(torch.equal(a, b) for a, b in zip(again, eager[(rep + 1) % 4]))
+                torch.cuda.synchronize()
+        assert g.replays == 12
+    finally:
+        DynamicLinear.prof = old
