@@ -27,6 +27,7 @@ struct GemmArgs {
     int M, N, K;
     void* partial;            // split-K: [splits][M][N] fp32 / int32 partial sums, else null
     int splits;               // number of K splits (1 = none)
+    int n_begin, n_cols;      // output columns this launch covers (a multiple of the tile width unless it ends at N)
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
@@ -309,10 +310,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
-    const int TM_ = (M + BM - 1) / BM, TN_ = (N + BN - 1) / BN;
+    const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + BN - 1) / BN;
     const int split = blockIdx.x / (TM_ * TN_);
     tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
     const long a_row_bytes = I8 ? (long)K : (long)K * 2;
     const int KT_all = (int)(a_row_bytes >> 7);
     const int kt_per = (KT_all + p.splits - 1) / p.splits;
@@ -570,10 +571,10 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
-    const int TM_ = (M + BM - 1) / BM, TN_ = (N + BN - 1) / BN;
+    const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + BN - 1) / BN;
     const int split = blockIdx.x / (TM_ * TN_);
     tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
     const long row_bytes = I8 ? (long)K : (long)K * 2;
     const int T_all = (int)(row_bytes >> 6);                // 64-byte stages along K
     const int t_per = (T_all + p.splits - 1) / p.splits;
@@ -776,8 +777,11 @@ static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
 }
 
 template <int KIND, int BM, int BN, bool TILED>
-static int launch_gemm(const GemmArgs& a_in, hipStream_t st) {
+static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
+    a.n_begin = n_begin;
+    a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
+    const bool whole = (a.n_begin == 0 && a.n_cols == a.N);
     constexpr bool DIRECT = (KIND == KIND_F16 || KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     constexpr int NS = 4;
     constexpr size_t lds = DIRECT ? (size_t)NS * (BM + BN) * 64 : 2 * (size_t)(BM + BN) * 128;
@@ -795,12 +799,12 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st) {
     const bool i8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     // units the kernels split K in: 128-byte k-tiles (register-staged) or 64-byte stages (direct)
     const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
-    a.splits = pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units);
+    a.splits = whole ? pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units) : 1;
     a.partial = a.splits > 1 ? g_workspace : nullptr;
 #ifdef KMI_DBG_TIMING
     a.partial = g_workspace;
 #endif
-    const dim3 grid(((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
+    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
         const long quads = (long)a.M * a.N / 4;
@@ -821,6 +825,20 @@ extern "C" int kmi_gemm_pick_tile(int M, int N) { return pick_tile(M, N); }
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
     const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N);
+    if (tile == 256 && force_tile == 0) {
+        // Round quantisation: TM x TN tiles run in rounds of 256 (one workgroup per CU).  When the last
+        // round would be at most ~60 % full, the columns it would cover are run with the 128x128 tile
+        // instead (four times as many workgroups of a quarter of the work, two per CU), so the tail costs
+        // about half a round; the two launches cover disjoint column ranges split at a multiple of 256.
+        const int TM = (a.M + 255) / 256, TN = (a.N + 255) / 256;
+        const int tiles = TM * TN, rem = tiles % 256;
+        const int head_cols = ((tiles - rem) / TM);          // column tiles that make up whole rounds
+        if (tiles > 256 && rem > 0 && head_cols > 0 && (TN - head_cols) * TM <= 160) {
+            const int rc = launch_gemm<KIND, 256, 256, TILED>(a, st, 0, head_cols * 256);
+            if (rc != KMI_OK) return rc;
+            return launch_gemm<KIND, 128, 128, TILED>(a, st, head_cols * 256, a.N - head_cols * 256);
+        }
+    }
     switch (tile) {
         case 256: return launch_gemm<KIND, 256, 256, TILED>(a, st);
         case 128: return launch_gemm<KIND, 128, 128, TILED>(a, st);
@@ -855,42 +873,42 @@ extern "C" int kmi_gemm_w4a16(void* out, const void* x, const void* qweight, con
                               const void* bias, int M, int N, int K, int G, void* stream) {
     if (G != 128) return kmi_set_error(KMI_E_GROUP, "kmi_gemm_w4a16: group size %d unsupported (128 only)", G);
     if (!scales || !szeros) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w4a16: NULL scale table");
-    GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w4a16", KIND_W4A16, false)
 }
 
 extern "C" int kmi_gemm_w8a16(void* out, const void* x, const void* w8, const void* wscales, const void* bias,
                               int M, int N, int K, void* stream) {
     if (!wscales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a16: NULL wscales");
-    GemmArgs a{out, x, w8, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, x, w8, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a16", KIND_W8A16, false)
 }
 
 extern "C" int kmi_gemm_w8a8(void* out, const void* a8, const void* w8, const void* wscales, const void* ascales,
                              const void* bias, int M, int N, int K, void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8: NULL scale vector");
-    GemmArgs a{out, a8, w8, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, a8, w8, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8", KIND_W8A8, false)
 }
 
 extern "C" int kmi_gemm_w8a8_acc_i32(void* acc, const void* a8, const void* w8, int M, int N, int K, void* stream) {
-    GemmArgs a{acc, a8, w8, nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, nullptr, 1};
+    GemmArgs a{acc, a8, w8, nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8_acc_i32", KIND_W8A8_ACC, false)
 }
 
 extern "C" int kmi_gemm_f16(void* out, const void* x, const void* w16, const void* bias, int M, int N, int K, void* stream) {
-    GemmArgs a{out, x, w16, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, x, w16, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_f16", KIND_F16, false)
 }
 
 extern "C" int kmi_gemm_w8a8_tiled(void* out, const void* a8, const void* w8t, const void* wscales, const void* ascales,
                                    const void* bias, int M, int N, int K, void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8_tiled: NULL scale vector");
-    GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8_tiled", KIND_W8A8, true)
 }
 
 extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, const void* bias, int M, int N, int K, void* stream) {
-    GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1};
+    GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_f16_tiled", KIND_F16, true)
 }

@@ -368,3 +368,40 @@ def test_prep_w8a8_equals_separate_kernels(ops, tiled, M, N, K):
     # and against the oracle directly
     a_o, sc_o = O.quant_act_i8(x.cpu().numpy())
     assert np.array_equal(a_f.cpu().numpy(), a_o)
+
+
+@pytest.mark.gpu
+def test_gemm_tail_round_split(ops):
+    """More than 256 tiles of 256x256 with a thin last round: the automatic choice runs the tail columns with
+    the 128x128 tile in a second launch.  Integer results must equal the single-tile runs bit for bit and the
+    oracle on sampled rows; the fp16-output lanes must equal their single-tile runs too."""
+    M, N, K = 4096, 6144, 256                      # 16 x 24 = 384 tiles -> head 16 column tiles, tail 8
+    rng = np.random.default_rng(5)
+    a8 = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    w8 = rng.integers(-128, 128, size=(N, K)).astype(np.int8)
+    a8d, w8d = dev(a8), dev(w8)
+    acc_auto = ops.w8a8_gemm_acc_i32(a8d, w8d, N)
+    ops.force_gemm_tile(128)
+    try:
+        acc_128 = ops.w8a8_gemm_acc_i32(a8d, w8d, N)
+    finally:
+        ops.force_gemm_tile(0)
+    assert torch.equal(acc_auto, acc_128)
+    rows = np.r_[0:8, 2040:2056, M - 8:M]
+    assert np.array_equal(host(acc_auto)[rows], O.gemm_i8_acc(a8[rows], w8))
+    # scaled fp16 output with bias, and the fp16 GEMM, across the seam at column 4096
+    ws = dev(rng.random(N).astype(np.float16)); as_ = dev(rng.random(M).astype(np.float16))
+    bias = dev(rng.standard_normal(N).astype(np.float16))
+    out_auto = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    out_256 = torch.empty_like(out_auto)
+    ops.w8a8_gemm_forward(a8d, w8d, ws, as_, out_auto, bias=bias)
+    x = dev(rng.standard_normal((M, K)).astype(np.float16)); w16 = dev((rng.standard_normal((N, K)) * 0.05).astype(np.float16))
+    f_auto = ops.f16_gemm_forward(x, w16, N)
+    ops.force_gemm_tile(256)
+    try:
+        ops.w8a8_gemm_forward(a8d, w8d, ws, as_, out_256, bias=bias)
+        f_256 = ops.f16_gemm_forward(x, w16, N)
+    finally:
+        ops.force_gemm_tile(0)
+    assert torch.equal(out_auto, out_256)
+    assert torch.equal(f_auto, f_256)
