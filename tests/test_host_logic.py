@@ -112,3 +112,22 @@ def test_temp_cache_is_bounded_and_reuses():
     with pytest.raises(MemoryError):
         c.get(3, 'f16', (4, 256), torch.float16, 'cpu')
     assert c.capacity <= 1024
+
+
+def test_committed_mi355x_tables_load_and_have_three_regimes():
+    """Every table shipped under kairos_amd/prof/ has the reference's file format and the small-M / mid-M /
+    large-M structure (same schema as the reference's prof_llama / prof_qwen files)."""
+    import glob
+    import json
+    import os
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "kairos_amd", "prof")
+    files = sorted(glob.glob(os.path.join(root, "*", "seg_perf_list.pt")))
+    assert len(files) >= 3
+    for f in files:
+        table = json.load(open(f))
+        assert len(table) == 4
+        for segs in table:
+            edges = [s[0] for s in segs]
+            assert edges == sorted(edges) and all(isinstance(e, int) for e in edges)
+            assert all(isinstance(s[1], str) and isinstance(s[2], float) for s in segs)
+            assert segs[0][1] == "w4a16_gemv" and segs[-1][1] == "w8a8"
