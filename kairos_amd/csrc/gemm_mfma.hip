@@ -8,8 +8,10 @@
 // 128 int8).  In LDS a row is eight 16-byte chunks; chunk c of row r is stored at c ^ ((r>>1)&7),
 // which makes both the 16-byte staging writes and the MFMA fragment reads (32 consecutive rows, one
 // logical chunk) bank-conflict free.  256 threads = 2x2 waves; each wave owns a (BM/2)x(BN/2) block
-// of 32x32 accumulator tiles.  Global loads for k-tile t+1 are issued before the MFMAs of k-tile t
-// and written to the other LDS stage afterwards: one barrier per k-tile.
+// of 32x32 accumulator tiles.  That is the register-staged kernel (gemm_kernel: W4A16, W8A16), which
+// keeps two k-tiles in flight in two register sets and writes them to the other of two LDS stages:
+// one barrier per k-tile.  The operand-copy kinds (F16, W8A8) use gemm_direct_kernel further down:
+// direct-to-LDS loads, four 64-byte stages.
 #include "kmi_common.h"
 #include <type_traits>
 
@@ -537,10 +539,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 // =================================================================================================
 // Direct-to-LDS variant for the operand-copy kinds (KIND_F16, KIND_W8A8, KIND_W8A8_ACC).
 //
-// A lone workgroup of the register-staged kernel above spends ~1.9 us per 128-byte k-tile, against
-// 0.85 us of MFMA work: with one workgroup per CU the only way to cover the ~1.6 us global-load
-// latency is to keep several k-tiles in flight, and registers cannot hold them.  Here global loads
-// write LDS directly (global_load_lds_dwordx4: the 64 lanes of a wave fill one contiguous KiB), so
+// With one workgroup per CU (a 256x256 tile needs all 512 VGPRs) only LDS can hold enough bytes in
+// flight to cover the global-load latency: registers cannot hold several k-tiles.  Here global loads
+// write LDS directly (buffer_load_dwordx4 ... lds: the 64 lanes of a wave fill one contiguous KiB), so
 // the spare LDS stages ARE the in-flight buffer: NS stages of (BM+BN) rows x 64 bytes, loads issued
 // NS-1 stages ahead, one barrier per stage.
 //
