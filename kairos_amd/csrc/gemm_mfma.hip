@@ -32,6 +32,9 @@ struct GemmArgs {
     int n_begin, n_cols;      // output columns this launch covers (a multiple of the tile width unless it ends at N)
 };
 
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
+
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 // int8 x4 -> two fp16 pairs, exactly: flip the sign bit (b+128 in 0..255), splice each byte under
@@ -537,6 +540,226 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 }
 
 // =================================================================================================
+// W4A16 for M up to a few hundred rows: wave-private weights.
+//
+// With so few rows the register-staged kernel above is bound by instruction issue, not by MFMA or
+// memory: every weight passes through LDS (a write and two fragment reads) and one wave per SIMD
+// serialises decode, LDS and load issue.  Here a workgroup tile is BM rows x 128 columns and each
+// wave owns 32 of the columns for itself, so its weights never touch LDS: lane (n = lane%32,
+// h = lane/32) loads the 16-byte chunk h of row n of the 64-wide k-tile (32 weights), decodes its four
+// 8-weight planes exactly as the converters do, and trades two of them with lane n of the other half
+// (v_permlane32_swap) so that each half holds the k-blocks its MFMA operand position needs:
+//   lower lanes  k 0-7, 32-39, 16-23, 48-55      upper lanes  k 8-15, 40-47, 24-31, 56-63
+// i.e. MFMA j of the four per k-tile covers the 16-wide k-step {0, 2, 1, 3}[j]; the activation fragment
+// of that k-step is read from LDS.  Only the activations are staged (direct-to-LDS loads, PF+1 stages),
+// shared by the four column waves.  The workgroup has KH such wave quartets; quartet q takes k-tiles
+// q, q+KH, ... and the quartets' accumulators meet in LDS at the end (fixed order).  A scale and a
+// scaled zero arrive in ONE load (lower lanes fetch the scale, upper lanes the zero of the same column)
+// and are spread with one more swap.  Per wave and k-tile: BM/32 + 2 load instructions, no LDS write.
+template <int BM, int KH, int PF>
+__global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int FM = BM / 32;
+    constexpr int NSA = PF + 1;                      // activation stages per quartet
+    constexpr int A_STAGE = BM * 128;                // bytes: BM rows x 64 fp16
+    constexpr int A_LD = BM / 32;                    // direct loads per wave and k-tile
+    constexpr int OPS = A_LD + 2;                    // load instructions per wave and k-tile
+    static_assert(BM == 32 || BM == 64 || BM == 128, "row tiles of 32, 64 or 128");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wc = wave & 3, kq = wave >> 2;
+    const int M = p.M, N = p.N, K = p.K;
+    const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + 127) / 128;
+    const int split = blockIdx.x / (TM_ * TN_);
+    int tm, tn;
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
+    const int m0 = tm * BM, n0 = p.n_begin + tn * 128;
+    const int KT_all = K >> 6;                       // 64-wide k-tiles
+    const int kt_per = (((KT_all + p.splits - 1) / p.splits) + KH - 1) / KH * KH;
+    const int kt0 = split * kt_per;
+    const int KT = (kt0 + kt_per <= KT_all) ? kt_per : KT_all - kt0;     // multiple of KH (host checks K)
+    const int T = KT / KH;                           // k-tiles of this quartet: kt0 + kq + j*KH
+
+    f16_t acc[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+
+    // ---- sources
+    char* ring = smem + kq * (NSA * A_STAGE);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.a), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.b), 0, -1, 0x00020000);
+    uint32_t voff_a[A_LD];
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+        const int row = 8 * (wc + 4 * i) + (lane >> 3), pc = lane & 7;
+        const int c = pc ^ ((row >> 1) & 7);
+        int m = m0 + row;
+        m = m < M ? m : M - 1;
+        voff_a[i] = (uint32_t)((long)m * K * 2 + c * 16);
+    }
+    const int hl = lane >> 5;
+    int ncol = n0 + wc * 32 + (lane & 31);
+    ncol = ncol < N ? ncol : N - 1;                  // ragged last strip: clamp loads, stores are masked
+    const uint32_t voff_b = (uint32_t)((long)(ncol >> 2) * K * 2 + (ncol & 3) * 32 + hl * 16);
+    const half_t* szp = (hl ? p.szeros : p.scales) + ncol;
+
+    u4_t rb[PF];
+    half_t rsz[PF];
+    auto issue = [&](auto set, int j_req) {          // loads of this quartet's j-th k-tile
+        constexpr int S = decltype(set)::value;
+        const int j = j_req < T ? j_req : T - 1;     // past the end: harmless reloads, never used
+        const int g = kt0 + kq + j * KH;
+        char* dst = ring + (j_req % NSA) * A_STAGE + wc * 1024;
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, voff_a[i], (uint32_t)g * 128u, 0, 0);
+        rb[S] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b, (uint32_t)g * 128u, 0);
+        rsz[S] = szp[(long)(g >> 1) * N];
+    };
+
+    // Wait until the loads of the k-tile about to be used have landed (the PF-1 younger k-tiles may stay
+    // in flight: OPS instructions each, issued in whole groups), then meet the other waves: after the
+    // barrier that k-tile's activations are complete and the previous one's stage is free.
+#define KMI_WP_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+    auto tile_barrier = [&]() {
+        constexpr int KEEP = (PF - 1) * OPS;
+        static_assert(KEEP == 6 || KEEP == 8 || KEEP == 9 || KEEP == 12 || KEEP == 18, "no immediate for this depth");
+        if constexpr (KEEP == 6) KMI_WP_BARRIER(6);
+        else if constexpr (KEEP == 8) KMI_WP_BARRIER(8);
+        else if constexpr (KEEP == 9) KMI_WP_BARRIER(9);
+        else if constexpr (KEEP == 12) KMI_WP_BARRIER(12);
+        else KMI_WP_BARRIER(18);
+    };
+
+    const int fr = lane & 31;
+    auto body = [&](auto set, int j) {
+        constexpr int S = decltype(set)::value;
+        tile_barrier();
+        // all activation fragments of the k-tile first: the decode below covers the LDS round trip
+        const char* st = ring + (j % NSA) * A_STAGE;
+        u4_t fa[4][FM];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int i = 0; i < FM; ++i) fa[ks][i] = *reinterpret_cast<const u4_t*>(st + lds_off(i * 32 + fr, 2 * ks + hl));
+        // decode this lane's chunk: planes 0..3 = k 8a..8a+7 of its 32-wide half of the k-tile
+        const uint32_t own = (uint32_t)__builtin_bit_cast(unsigned short, rsz[S]);
+        const auto sw = __builtin_amdgcn_permlane32_swap(own, own, false, false);
+        const uint32_t sbits = sw[0], zbits = sw[1];          // scale / scaled zero in every lane
+        const h2_t s2 = as_h2(sbits | (sbits << 16)), z2 = as_h2(zbits | (zbits << 16));
+        const u4_t raw = rb[S];
+        u4_t pl[4];
+        pl[0] = __builtin_bit_cast(u4_t, dequant_nibble<0>(raw, s2, z2));
+        pl[1] = __builtin_bit_cast(u4_t, dequant_nibble<1>(raw, s2, z2));
+        pl[2] = __builtin_bit_cast(u4_t, dequant_nibble<2>(raw, s2, z2));
+        pl[3] = __builtin_bit_cast(u4_t, dequant_nibble<3>(raw, s2, z2));
+        // lower lanes keep planes 0, 2 of both chunks, upper lanes planes 1, 3
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t a0 = pl[0][w], a1 = pl[1][w], a2 = pl[2][w], a3 = pl[3][w];
+            const auto x01 = __builtin_amdgcn_permlane32_swap(a0, a1, false, false);
+            const auto x23 = __builtin_amdgcn_permlane32_swap(a2, a3, false, false);
+            pl[0][w] = x01[0]; pl[1][w] = x01[1];
+            pl[2][w] = x23[0]; pl[3][w] = x23[1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue(set, j + PF);                                  // refills the registers just consumed
+        __builtin_amdgcn_sched_barrier(0);
+        // pl[jj] covers k-step {0, 2, 1, 3}[jj]
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int ks = (jj == 1) ? 2 : (jj == 2) ? 1 : jj;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, pl[jj]), __builtin_bit_cast(h8_t, fa[ks][i]),
+                                                                acc[i], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- pipeline: PF k-tiles in flight per wave
+    {
+        int j = 0;
+        auto prime = [&](auto set) { issue(set, j); ++j; __builtin_amdgcn_sched_barrier(0); };
+        prime(std::integral_constant<int, 0>{});
+        if constexpr (PF > 1) prime(std::integral_constant<int, 1>{});
+        if constexpr (PF > 2) prime(std::integral_constant<int, 2>{});
+        if constexpr (PF > 3) prime(std::integral_constant<int, 3>{});
+        static_assert(PF >= 2 && PF <= 4, "prefetch depth 2..4");
+    }
+    int j = 0;
+    for (; j + PF <= T; j += PF) {
+        body(std::integral_constant<int, 0>{}, j);
+        if constexpr (PF > 1) body(std::integral_constant<int, 1>{}, j + 1);
+        if constexpr (PF > 2) body(std::integral_constant<int, 2>{}, j + 2);
+        if constexpr (PF > 3) body(std::integral_constant<int, 3>{}, j + 3);
+    }
+    if (j < T) { body(std::integral_constant<int, 0>{}, j); ++j; }
+    if constexpr (PF > 2) if (j < T) { body(std::integral_constant<int, 1>{}, j); ++j; }
+    if constexpr (PF > 3) if (j < T) { body(std::integral_constant<int, 2>{}, j); ++j; }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // no load outlives its stage
+#undef KMI_WP_BARRIER
+
+    // ---- the quartets' partial sums meet in LDS, added to quartet 0 in quartet order
+    if constexpr (KH > 1) {
+        float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+        for (int q = 1; q < KH; ++q) {
+            if (kq == q) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) red[((wc * FM + i) * 16 + e) * 64 + lane] = acc[i][e];
+            }
+            __syncthreads();
+            if (kq == 0) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][e] += red[((wc * FM + i) * 16 + e) * 64 + lane];
+            }
+            __syncthreads();
+        }
+        if (kq != 0) return;
+    }
+
+    // ---- output: lane (row = lane%32, hl) holds columns 8g + 4hl + (0..3) of its wave's 32
+    const int nw = n0 + wc * 32;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = m0 + i * 32 + fr;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = nw + 8 * g + 4 * hl;
+            if (m < M && n < N) {
+                if (p.splits > 1) {
+                    u4_t v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float f = acc[i][4 * g + r];
+                        v[r] = __builtin_bit_cast(uint32_t, f);
+                    }
+                    *reinterpret_cast<u4_t*>(static_cast<uint32_t*>(p.partial) + (long)split * M * N + (long)m * N + n) = v;
+                } else {
+                    half_t h[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        h[r] = (half_t)acc[i][4 * g + r];
+                        if (p.bias) h[r] = (half_t)((float)h[r] + (float)p.bias[n + r]);
+                    }
+                    *reinterpret_cast<h4_t*>(static_cast<half_t*>(p.out) + (long)m * N + n) = h4_t{h[0], h[1], h[2], h[3]};
+                }
+            }
+        }
+    }
+#endif
+}
+
+// =================================================================================================
 // Direct-to-LDS variant for the operand-copy kinds (KIND_F16, KIND_W8A8, KIND_W8A8_ACC).
 //
 // With one workgroup per CU (a 256x256 tile needs all 512 VGPRs) only LDS can hold enough bytes in
@@ -550,8 +773,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 // direct load puts lane l's data at slot l, the swizzle is applied on the global side: lane l
 // fetches the chunk that belongs in slot l.  The tiled weight layout ([N/128][K-stages][128][64 B],
 // already swizzled) makes the B side a straight 8 KiB copy per 128-row strip.
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
 template <int KIND, int BM, int BN, bool TILED_B, int NS>
 __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
@@ -814,6 +1035,45 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, in
     return KMI_OK;
 }
 
+// Launch of the wave-private-weights kernel (W4A16, small M).  K is split over KH wave quartets inside the
+// workgroup and, when the tiles alone leave CUs idle, over workgroups as well (partials + reduce kernel).
+template <int BM>
+static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
+    GemmArgs a = a_in;
+    constexpr int KH = 2, PF = 4;
+    constexpr size_t lds = (size_t)KH * (PF + 1) * BM * 128;
+    void (*fn)(GemmArgs) = gemm_w4a16_wp_kernel<BM, KH, PF>;
+    static thread_local bool raised = false;
+    if (lds > 64 * 1024 && !raised) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return kmi_set_error(KMI_E_LAUNCH, "gemm: cannot raise the dynamic LDS limit to %zu bytes", lds);
+        raised = true;
+    }
+    a.n_begin = 0;
+    a.n_cols = a.N;
+    const int tiles = ((a.M + BM - 1) / BM) * ((a.N + 127) / 128);
+    const int kt_all = a.K / 64;
+    int s = g_force_splits > 0 ? g_force_splits : 256 / tiles;
+    if (s > 8) s = 8;
+    if (s > kt_all / 16) s = kt_all / 16;                       // at least 16 k-tiles (8 per quartet) per split
+    const size_t per = (size_t)a.M * a.N * 4;
+    if (g_workspace == nullptr || per == 0) s = 1;
+    else if ((size_t)s * per > g_workspace_bytes) s = (int)(g_workspace_bytes / per);
+    if (s < 1) s = 1;
+    if (s > 1) {                                                 // whole quartet rounds per split, no empty split
+        const int per_split = ((kt_all + s - 1) / s + KH - 1) / KH * KH;
+        s = (kt_all + per_split - 1) / per_split;
+    }
+    a.splits = s;
+    a.partial = s > 1 ? g_workspace : nullptr;
+    hipLaunchKernelGGL(fn, dim3(tiles * s), dim3(256 * KH), lds, st, a);
+    if (s > 1) {
+        const long quads = (long)a.M * a.N / 4;
+        hipLaunchKernelGGL(splitk_reduce_kernel<KIND_W4A16>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, a);
+    }
+    return KMI_OK;
+}
+
 // Tile choice: the largest tile that still yields about one workgroup per CU.
 static int pick_tile(int M, int N) {
     auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -822,6 +1082,20 @@ static int pick_tile(int M, int N) {
     return 64;
 }
 extern "C" int kmi_gemm_pick_tile(int M, int N) { return pick_tile(M, N); }
+
+// Rows per tile of the wave-private-weights W4A16 kernel, or 0 when the register-staged kernel runs.
+// Measured on MI355X (Llama-3-8B shapes): the wave-private kernel wins while its tiles fit one round over
+// the CUs; beyond that the register-staged kernel's larger tiles amortise the decode.
+static int pick_wp_rows(int M, int N) {
+    if (M > 512) return 0;
+    const long strips = (N + 127) / 128;
+    if (M <= 32) return 32;
+    if (M <= 64) return 64;
+    if (((M + 63) / 64) * strips <= 256) return 64;
+    if (((M + 127) / 128) * strips <= 192) return 128;
+    return 0;
+}
+extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N) { return pick_wp_rows(M, N); }
 
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
@@ -838,6 +1112,19 @@ static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
             const int rc = launch_gemm<KIND, 256, 256, TILED>(a, st, 0, head_cols * 256);
             if (rc != KMI_OK) return rc;
             return launch_gemm<KIND, 128, 128, TILED>(a, st, head_cols * 256, a.N - head_cols * 256);
+        }
+    }
+    if constexpr (KIND == KIND_W4A16) {
+        // selectors 1032 / 1064 / 1128 force the wave-private-weights kernel with 32 / 64 / 128 rows per tile
+        if (tile == 1032) return launch_w4a16_wp<32>(a, st);
+        if (tile == 1064) return launch_w4a16_wp<64>(a, st);
+        if (tile == 1128) return launch_w4a16_wp<128>(a, st);
+        if (force_tile == 0) {
+            switch (pick_wp_rows(a.M, a.N)) {
+                case 32: return launch_w4a16_wp<32>(a, st);
+                case 64: return launch_w4a16_wp<64>(a, st);
+                case 128: return launch_w4a16_wp<128>(a, st);
+            }
         }
     }
     switch (tile) {

@@ -405,3 +405,39 @@ def test_gemm_tail_round_split(ops):
         ops.force_gemm_tile(0)
     assert torch.equal(out_auto, out_256)
     assert torch.equal(f_auto, f_256)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,sel,splits", [
+    (5, 128, 128, 1032, 0), (32, 256, 512, 1032, 0), (64, 256, 512, 1064, 0), (33, 384, 1024, 1064, 0),
+    (64, 128, 4096, 1064, 2), (100, 256, 512, 1064, 0), (128, 256, 1024, 1128, 0), (48, 132, 256, 1064, 0),
+    (17, 256, 2048, 1032, 3), (300, 384, 512, 1128, 0), (1, 128, 14336, 1032, 0)])
+def test_gemm_w4a16_wave_private(ops, M, N, K, sel, splits):
+    """The small-M W4A16 variant (weights decoded in registers by the wave that owns their columns, quartets
+    splitting K inside the workgroup, optional split over workgroups) against the oracle, with and without
+    bias, ragged N included; repeated calls give the same bits."""
+    p = prep(N, K, seed=N + K)
+    x = O.synth_acts(M, K, seed=M)
+    ref = O.gemm_w4a16(x, p["qweight"], p["scales"], p["scaled_zeros"])
+    bias = np.random.default_rng(1).standard_normal(N).astype(np.float16)
+    args = (dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]))
+    ops.force_gemm_tile(sel)
+    ops.force_gemm_splits(splits)
+    try:
+        out = ops.gemm_forward(*args)
+        again = ops.gemm_forward(*args)
+        outb = ops.gemm_forward(*args, bias=dev(bias))
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert O.max_abs_rel(host(out), ref) < 2e-3
+    assert torch.equal(out, again)
+    refb = (host(out).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)   # fp16 add after rounding
+    assert_same_bits(host(outb), refb)
+
+
+@pytest.mark.gpu
+def test_gemm_w4a16_variant_choice(ops):
+    assert ops.gemm_w4a16_wp_rows(1, 4096) == 32 and ops.gemm_w4a16_wp_rows(64, 28672) == 64
+    assert ops.gemm_w4a16_wp_rows(256, 6144) == 64 and ops.gemm_w4a16_wp_rows(512, 6144) == 128
+    assert ops.gemm_w4a16_wp_rows(256, 28672) == 0 and ops.gemm_w4a16_wp_rows(1024, 4096) == 0
