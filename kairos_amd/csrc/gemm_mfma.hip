@@ -539,6 +539,35 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
 }
 
+// dequant_nibble with the masks and the exponent pattern held in registers, so that mask-and-splice is one
+// v_and_or_b32 instead of two literal-operand instructions (a VOP3 cannot take literals on gfx9).  Same
+// arithmetic, same bits.
+struct NibConsts { uint32_t mask_lo, mask_hi, magic; };
+__device__ __forceinline__ NibConsts nib_consts() {
+    NibConsts c{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+    asm volatile("" : "+s"(c.mask_lo), "+s"(c.mask_hi), "+v"(c.magic));      // opaque: keeps them out of the instructions
+    return c;
+}
+template <int A>
+__device__ __forceinline__ h8_t dequant_nibble_r(const u4_t& u, h2_t s2, h2_t z2, const NibConsts& c) {
+    const h2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    const h2_t k16th = {(half_t)0.0625f, (half_t)0.0625f};
+    const h2_t km64 = {(half_t)-64.0f, (half_t)-64.0f};
+    h2_t r[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const uint32_t w = (A >= 2) ? (u[t] >> 8) : u[t];
+        h2_t q;
+        if constexpr (A & 1) q = pk_fma(as_h2((w & c.mask_hi) | c.magic), k16th, km64);
+        else q = as_h2((w & c.mask_lo) | c.magic) - k1024;
+        r[t] = pk_fma(q, s2, z2);
+    }
+    h8_t o;
+    o[0] = r[0][0]; o[1] = r[0][1]; o[2] = r[1][0]; o[3] = r[1][1];
+    o[4] = r[2][0]; o[5] = r[2][1]; o[6] = r[3][0]; o[7] = r[3][1];
+    return o;
+}
+
 // =================================================================================================
 // W4A16 for M up to a few hundred rows: wave-private weights.
 //
@@ -636,6 +665,7 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
     };
 
     const int fr = lane & 31;
+    const NibConsts nc = nib_consts();
     auto body = [&](auto set, int j) {
         constexpr int S = decltype(set)::value;
         tile_barrier();
@@ -653,10 +683,10 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         const h2_t s2 = as_h2(sbits | (sbits << 16)), z2 = as_h2(zbits | (zbits << 16));
         const u4_t raw = rb[S];
         u4_t pl[4];
-        pl[0] = __builtin_bit_cast(u4_t, dequant_nibble<0>(raw, s2, z2));
-        pl[1] = __builtin_bit_cast(u4_t, dequant_nibble<1>(raw, s2, z2));
-        pl[2] = __builtin_bit_cast(u4_t, dequant_nibble<2>(raw, s2, z2));
-        pl[3] = __builtin_bit_cast(u4_t, dequant_nibble<3>(raw, s2, z2));
+        pl[0] = __builtin_bit_cast(u4_t, dequant_nibble_r<0>(raw, s2, z2, nc));
+        pl[1] = __builtin_bit_cast(u4_t, dequant_nibble_r<1>(raw, s2, z2, nc));
+        pl[2] = __builtin_bit_cast(u4_t, dequant_nibble_r<2>(raw, s2, z2, nc));
+        pl[3] = __builtin_bit_cast(u4_t, dequant_nibble_r<3>(raw, s2, z2, nc));
         // lower lanes keep planes 0, 2 of both chunks, upper lanes planes 1, 3
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
