@@ -441,3 +441,30 @@ def test_gemm_w4a16_variant_choice(ops):
     assert ops.gemm_w4a16_wp_rows(1, 4096) == 32 and ops.gemm_w4a16_wp_rows(64, 28672) == 64
     assert ops.gemm_w4a16_wp_rows(256, 6144) == 64 and ops.gemm_w4a16_wp_rows(512, 6144) == 128
     assert ops.gemm_w4a16_wp_rows(256, 28672) == 0 and ops.gemm_w4a16_wp_rows(1024, 4096) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(48, 28672, 4096), (200, 4096, 14336)])
+def test_gemm_w4a16_variants_agree_at_full_size(ops, M, N, K):
+    """At BASELINE sizes the oracle is too slow; the two W4A16 GEMM variants (wave-private, register-staged) and
+    the small-M kernel are independent implementations of the same product and must agree within the fp16
+    tolerance on random packed weights."""
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    qw = torch.randint(-32768, 32767, (N // 4, K), device="cuda", dtype=torch.int16, generator=g)
+    Gp = (K // 128 + 7) // 8 * 8
+    s = (torch.rand((Gp, N), device="cuda", generator=g) * 0.01 + 0.002).to(torch.float16)
+    z = (-(s.float() * 7.5)).to(torch.float16)
+    x = torch.randn((M, K), device="cuda", generator=g).to(torch.float16)
+    auto = ops.gemm_forward(x, qw, s, z)
+    assert ops.gemm_w4a16_wp_rows(M, N) in (64, 128)
+    ops.force_gemm_tile(64)
+    try:
+        staged = ops.gemm_forward(x, qw, s, z)
+    finally:
+        ops.force_gemm_tile(0)
+    a, b = auto.float(), staged.float()
+    scale = b.abs().max()
+    assert ((a - b).abs().max() / scale).item() < 2e-3
+    if M <= 64:
+        v = ops.gemv_forward(x, qw, s, z, M, N, K, 128).float()
+        assert ((a - v).abs().max() / scale).item() < 2e-3
