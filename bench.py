@@ -27,8 +27,8 @@ M_GRID = [1 << i for i in range(13)]
 PEAK = {"hbm": 8.0e12, "f16": 2.5e15, "i8": 5.0e15}       # MI355X published: HBM3E B/s, dense MFMA op/s
 LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x")
 # HBM<->L2 bytes per launch of the dominant kernel, from the committed counter runs (profiles/
-# bench_llama3_8b_fetch_write_size.md): mean over the launches of one step, 2.0*FETCH_SIZE + WRITE_SIZE KiB.
-MEASURED_TRAFFIC = {"gemm_w8a8[256]": int((2.0 * 123224 + 66230) * 1024)}
+# bench_llama3_8b_fetch_write_size.md): mean over the calls of one step (tail launches included), 2.0*FETCH_SIZE + WRITE_SIZE KiB.
+MEASURED_TRAFFIC = {"gemm_w8a8[256]": int((2.0 * 137787 + 71171) * 1024)}
 G = 128
 
 
