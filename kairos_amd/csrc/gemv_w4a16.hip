@@ -46,11 +46,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
 
     const u4_t* wp[NT];
     int ncol[NT];
+    const half_t* szp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int n = n0 + nt * 16 + r16;
         n = n < N ? n : N - 1;                   // partial last strip: clamp loads, stores are masked
         ncol[nt] = n;
+        szp[nt] = ((lane >> 5) ? szeros : scales) + n;
         wp[nt] = qw + (long)(n >> 2) * kq + (n & 3) * 2 + (j & 1) + (j >> 1) * 8;
     }
     // Rows beyond M are not loaded at all (their lanes feed zeros): the texture path spends time per
@@ -71,7 +73,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
     const h8_t sixteenth = ones * (half_t)0.0625f;
     for (int c0 = wave; c0 < ngroups; c0 += NW * U) {
         u4_t u[U][NT];
-        half_t s[U][NT], z[U][NT];
+        half_t sz[U][NT];
         h8_t xa[U][MT][4];
 #pragma unroll
         for (int t = 0; t < U; ++t) {
@@ -80,8 +82,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 u[t][nt] = __builtin_nontemporal_load(wp[nt] + c * 16);
-                s[t][nt] = scales[(long)c * N + ncol[nt]];
-                z[t][nt] = szeros[(long)c * N + ncol[nt]];
+                sz[t][nt] = szp[nt][(long)c * N];              // lower half-wave: scale, upper: scaled zero
             }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
@@ -118,8 +119,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
                         lo8[w] = v8 & 0x000F000Fu;
                         hi8[w] = v8 & 0x00F000F0u;
                     }
-                    const float sc = (float)s[t][nt] * 16777216.0f;      // undo the 2^-24 of the subnormal encoding
-                    const float zc = (float)z[t][nt];
+                    // one load brought the scale to lanes 0-31 and the scaled zero to lanes 32-63 (same column:
+                    // it depends on lane%16 only); one swap gives every lane both
+                    const uint32_t own = (uint32_t)__builtin_bit_cast(unsigned short, sz[t][nt]);
+                    const auto both = __builtin_amdgcn_permlane32_swap(own, own, false, false);
+                    const float sc = (float)__builtin_bit_cast(half_t, (unsigned short)both[0]) * 16777216.0f;   // undo the 2^-24 of the subnormal encoding
+                    const float zc = (float)__builtin_bit_cast(half_t, (unsigned short)both[1]);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
                         f4_t pg = {0.f, 0.f, 0.f, 0.f};
