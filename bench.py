@@ -70,8 +70,8 @@ class Tracer:
 
     def begin(self, name, M, N, K):
         label = name
-        if name == "gemm_w4a16" and self.ops.gemm_w4a16_wp_rows(M, N):
-            label = f"{name}[wp{self.ops.gemm_w4a16_wp_rows(M, N)}]"
+        if name == "gemm_w4a16" and self.ops.gemm_w4a16_wp_rows(M, N, K):
+            label = f"{name}[wp{self.ops.gemm_w4a16_wp_rows(M, N, K)}]"
         elif name.startswith("gemm_"):
             label = f"{name}[{self.ops.gemm_tile_for(M, N)}]"
         ev = self.torch.cuda.Event(enable_timing=True)

@@ -139,10 +139,11 @@ void kmi_gemm_force_tile(int tile);
  * same stream (same results). */
 int kmi_gemm_pick_tile(int M, int N);
 
-/* Rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses for an M x N output (weights decoded
+/* Rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses for an M x N x K product (weights decoded
  * in registers by the wave that owns their columns), or 0 when the LDS-staged variant runs.  Forcing: tile
- * selectors 1032 / 1064 / 1128 in kmi_gemm_force_tile. */
-int kmi_gemm_w4a16_wp_rows(int M, int N);
+ * selectors 1032 / 1064 / 1128 (two wave quartets per workgroup) and 2032 / 2064 / 2128 (one) in
+ * kmi_gemm_force_tile. */
+int kmi_gemm_w4a16_wp_rows(int M, int N, int K);
 
 /* Optional scratch for split-K (used when the output tiles alone cannot fill the GPU, i.e. mid-sized
  * M): the calling thread registers a caller-owned device buffer; GEMM calls made by that thread then

@@ -1067,10 +1067,10 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, in
 
 // Launch of the wave-private-weights kernel (W4A16, small M).  K is split over KH wave quartets inside the
 // workgroup and, when the tiles alone leave CUs idle, over workgroups as well (partials + reduce kernel).
-template <int BM>
+template <int BM, int KH = 2>
 static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
     GemmArgs a = a_in;
-    constexpr int KH = 2, PF = 4;
+    constexpr int PF = 4;
     constexpr size_t lds = (size_t)KH * (PF + 1) * BM * 128;
     void (*fn)(GemmArgs) = gemm_w4a16_wp_kernel<BM, KH, PF>;
     static thread_local bool raised = false;
@@ -1113,19 +1113,25 @@ static int pick_tile(int M, int N) {
 }
 extern "C" int kmi_gemm_pick_tile(int M, int N) { return pick_tile(M, N); }
 
-// Rows per tile of the wave-private-weights W4A16 kernel, or 0 when the register-staged kernel runs.
-// Measured on MI355X (Llama-3-8B shapes): the wave-private kernel wins while its tiles fit one round over
-// the CUs; beyond that the register-staged kernel's larger tiles amortise the decode.
-static int pick_wp_rows(int M, int N) {
-    if (M > 512) return 0;
+// Variant of the wave-private-weights W4A16 kernel for an M x N x K product: rows per tile (0 = run the
+// register-staged kernel instead) and wave quartets per workgroup.  Measured on MI355X (Llama-3-8B shapes):
+// the wave-private kernel wins while its tiles fit one or two rounds over the CUs; 64-row tiles while they
+// fit one round, 128-row tiles beyond that or when K is long (the decode of a weight is then shared by twice
+// as many rows), a single quartet per workgroup once there are more tiles than CUs.
+struct WpChoice { int rows, quartets; };
+static WpChoice pick_wp(int M, int N, int K) {
+    if (M > 1024) return {0, 0};
     const long strips = (N + 127) / 128;
-    if (M <= 32) return 32;
-    if (M <= 64) return 64;
-    if (((M + 63) / 64) * strips <= 256) return 64;
-    if (((M + 127) / 128) * strips <= 192) return 128;
-    return 0;
+    const long tiles64 = ((M + 63) / 64) * strips, tiles128 = ((M + 127) / 128) * strips;
+    if (M <= 32) return {32, 2};
+    if (M <= 64) return {64, 2};
+    if (K >= 8192 && M > 128 && tiles128 <= 256) return {128, 2};
+    if (tiles64 <= 256) return {64, 2};
+    if (tiles128 <= 256) return {128, 2};
+    if (tiles128 <= 512) return {128, 1};
+    return {0, 0};
 }
-extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N) { return pick_wp_rows(M, N); }
+extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N, int K) { return pick_wp(M, N, K).rows; }
 
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
@@ -1149,12 +1155,15 @@ static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
         if (tile == 1032) return launch_w4a16_wp<32>(a, st);
         if (tile == 1064) return launch_w4a16_wp<64>(a, st);
         if (tile == 1128) return launch_w4a16_wp<128>(a, st);
+        if (tile == 2032) return launch_w4a16_wp<32, 1>(a, st);      // 2xxx: one wave quartet per workgroup
+        if (tile == 2064) return launch_w4a16_wp<64, 1>(a, st);
+        if (tile == 2128) return launch_w4a16_wp<128, 1>(a, st);
         if (force_tile == 0) {
-            switch (pick_wp_rows(a.M, a.N)) {
-                case 32: return launch_w4a16_wp<32>(a, st);
-                case 64: return launch_w4a16_wp<64>(a, st);
-                case 128: return launch_w4a16_wp<128>(a, st);
-            }
+            const WpChoice c = pick_wp(a.M, a.N, a.K);
+            if (c.rows == 32) return launch_w4a16_wp<32>(a, st);
+            if (c.rows == 64) return launch_w4a16_wp<64>(a, st);
+            if (c.rows == 128 && c.quartets == 2) return launch_w4a16_wp<128>(a, st);
+            if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, st);
         }
     }
     switch (tile) {

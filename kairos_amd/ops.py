@@ -195,9 +195,9 @@ def gemm_tile_for(M, N):
     return _lib.load().kmi_gemm_pick_tile(int(M), int(N))
 
 
-def gemm_w4a16_wp_rows(M, N):
-    """Rows per tile of the small-M W4A16 GEMM variant used for an M x N output (0: the LDS-staged variant)."""
-    return _lib.load().kmi_gemm_w4a16_wp_rows(int(M), int(N))
+def gemm_w4a16_wp_rows(M, N, K=4096):
+    """Rows per tile of the small-M W4A16 GEMM variant used for an M x N x K product (0: the LDS-staged variant)."""
+    return _lib.load().kmi_gemm_w4a16_wp_rows(int(M), int(N), int(K))
 
 
 _workspace = None

@@ -438,9 +438,10 @@ def test_gemm_w4a16_wave_private(ops, M, N, K, sel, splits):
 
 @pytest.mark.gpu
 def test_gemm_w4a16_variant_choice(ops):
-    assert ops.gemm_w4a16_wp_rows(1, 4096) == 32 and ops.gemm_w4a16_wp_rows(64, 28672) == 64
-    assert ops.gemm_w4a16_wp_rows(256, 6144) == 64 and ops.gemm_w4a16_wp_rows(512, 6144) == 128
-    assert ops.gemm_w4a16_wp_rows(256, 28672) == 0 and ops.gemm_w4a16_wp_rows(1024, 4096) == 0
+    assert ops.gemm_w4a16_wp_rows(1, 4096, 4096) == 32 and ops.gemm_w4a16_wp_rows(64, 28672, 4096) == 64
+    assert ops.gemm_w4a16_wp_rows(256, 6144, 4096) == 64 and ops.gemm_w4a16_wp_rows(512, 6144, 4096) == 128
+    assert ops.gemm_w4a16_wp_rows(256, 4096, 14336) == 128 and ops.gemm_w4a16_wp_rows(256, 28672, 4096) == 128
+    assert ops.gemm_w4a16_wp_rows(512, 28672, 4096) == 0 and ops.gemm_w4a16_wp_rows(2048, 4096, 4096) == 0
 
 
 @pytest.mark.gpu
@@ -456,7 +457,7 @@ def test_gemm_w4a16_variants_agree_at_full_size(ops, M, N, K):
     z = (-(s.float() * 7.5)).to(torch.float16)
     x = torch.randn((M, K), device="cuda", generator=g).to(torch.float16)
     auto = ops.gemm_forward(x, qw, s, z)
-    assert ops.gemm_w4a16_wp_rows(M, N) in (64, 128)
+    assert ops.gemm_w4a16_wp_rows(M, N, K) in (64, 128)
     ops.force_gemm_tile(64)
     try:
         staged = ops.gemm_forward(x, qw, s, z)
