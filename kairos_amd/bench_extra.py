@@ -78,9 +78,13 @@ def gemv70b(args):
         for M in (1, 2, 4, 8, 16, 32):
             x = _acts(M, K).to(dev)[None]
             us = _time(lambda i: layers[i % copies]._forward(x, M, COMP_TYPE_NAME["w4a16_gemv"]), 40)
+            # the other W4A16 lane (MFMA GEMM, wave-private weights at these M): what the LUT switches to
+            us_gemm = _time(lambda i: layers[i % copies]._forward(x, M, COMP_TYPE_NAME["w4a16_gemm"]), 40)
             b = N * K // 2 + 4 * (K // G) * N + 2 * M * K + 2 * M * N
+            best = min(us, us_gemm)
             rows.append({"shape": name, "N": N, "K": K, "M": M, "us": round(us, 2), "gbps": round(b / us / 1e3, 1),
-                         "hbm_frac": round(b / us / 1e-6 / HBM, 4)})
+                         "hbm_frac": round(b / us / 1e-6 / HBM, 4), "us_gemm_lane": round(us_gemm, 2),
+                         "hbm_frac_best_lane": round(b / best / 1e-6 / HBM, 4)})
             print(rows[-1], file=sys.stderr, flush=True)
         del layers
         torch.cuda.empty_cache()
