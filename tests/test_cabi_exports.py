@@ -49,6 +49,16 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_quant_act_i8(16, 16, 16, 4, 12, None) == -2
     assert lib.kmi_quant_act_i8(16, 16, 16, 0, 128, None) == 0        # empty batch is a no-op
     assert lib.kmi_gemm_f16(16, 16, 16, None, 0, 64, 128, None) == 0
+    # fused preparation launch: same rules as its two halves
+    assert lib.kmi_prep_w8a8(None, 0, 16, 16, 16, 4, 128, 128, 16, 16, 16, 2, None) == -1
+    assert lib.kmi_prep_w8a8(16, 0, 16, 16, 16, 4, 128, 64, 16, 16, 16, 2, None) == -3
+    assert lib.kmi_prep_w8a8(16, 1, 16, 16, 16, 4, 128, 128, 16, 16, 16, 2, None) == -2      # tiled needs N % 128 == 0
+    assert lib.kmi_prep_w8a8(16, 0, 16, 16, 16, 4, 128, 128, 8, 16, 16, 2, None) == -5
+    assert lib.kmi_prep_w8a8(16, 0, 16, 16, 16, 4, 128, 128, 16, 16, 16, -1, None) == -2
+    # variant choice of the W4A16 GEMM is host logic
+    assert lib.kmi_gemm_w4a16_wp_rows(16, 4096, 4096) == 32
+    assert lib.kmi_gemm_w4a16_wp_rows(4096, 4096, 4096) == 0
+    assert lib.kmi_gemm_pick_tile(4096, 4096) == 256 and lib.kmi_gemm_pick_tile(8, 4096) == 64
     assert lib.kmi_lut_get(None, 3) == -7
 
 
