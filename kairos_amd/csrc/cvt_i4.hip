@@ -9,7 +9,7 @@ __global__ __launch_bounds__(256) void cvt_i4_kernel(void* __restrict__ out, con
                                                      const half_t* __restrict__ scales,
                                                      const half_t* __restrict__ szeros, int N, int K,
                                                      long total_chunks) {
-    cvt_i4_body<OUT>((long)blockIdx.x * 256 + threadIdx.x, out, qw, scales, szeros, N, K, total_chunks);
+    cvt_i4_body<OUT>(cvt_chunk_of(blockIdx.x, threadIdx.x, N, K), out, qw, scales, szeros, N, K, total_chunks);
 }
 
 // tiled -> row-major (verification helper): one thread per 16-byte chunk

@@ -28,6 +28,25 @@ __device__ __forceinline__ u2_t h8_to_i8x8(h8_t v) {
     return o;
 }
 
+// Workgroup -> chunks, one chunk per thread.  Linear order (chunk = block*256 + thread) would make a workgroup
+// convert 32 k-blocks of ONE four-row block: its output is 32 runs of 256 bytes, 8 KiB apart in the tiled layout.
+// When the shape allows, a workgroup takes KMI_CVT_KB k-blocks of KMI_CVT_QB consecutive four-row blocks instead
+// (QB * KB = 32): reads are runs of KB*128 bytes, writes runs of 4*QB tile rows per k-block.
+#ifndef KMI_CVT_QB
+#define KMI_CVT_QB 8
+#endif
+#define KMI_CVT_KB (32 / KMI_CVT_QB)
+__device__ __forceinline__ long cvt_chunk_of(long block, int tid, int N, int K) {
+    const int per_quad = K >> 3;
+    if ((K % (64 * KMI_CVT_KB)) == 0 && (N % (4 * KMI_CVT_QB)) == 0) {
+        const long kb_groups = K / (64 * KMI_CVT_KB);
+        const long qg = block / kb_groups, kg = block - qg * kb_groups;
+        const int qd = tid / (8 * KMI_CVT_KB), rest = tid % (8 * KMI_CVT_KB);   // rest = (k-block, row, half)
+        return (qg * KMI_CVT_QB + qd) * per_quad + kg * (8 * KMI_CVT_KB) + rest;
+    }
+    return block * 256 + tid;
+}
+
 // Converts chunk i (32 weights of one row).  `out` layout by OUT; see the kernels' file header.
 template <int OUT>
 __device__ __forceinline__ void cvt_i4_body(long i, void* __restrict__ out, const u4_t* __restrict__ qw,

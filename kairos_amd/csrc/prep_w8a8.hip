@@ -16,7 +16,7 @@ __global__ __launch_bounds__(256) void prep_w8a8_kernel(void* __restrict__ w8, c
         quant_act_body<CPT>(blockIdx.x, a8, ascale, x, K);
         return;
     }
-    cvt_i4_body<OUT>((long)(blockIdx.x - M) * 256 + threadIdx.x, w8, qw, scales, szeros, N, K, total_chunks);
+    cvt_i4_body<OUT>(cvt_chunk_of((long)blockIdx.x - M, threadIdx.x, N, K), w8, qw, scales, szeros, N, K, total_chunks);
 }
 
 template <int OUT>
@@ -44,7 +44,7 @@ extern "C" int kmi_prep_w8a8(void* w8_out, int tiled, const void* qweight, const
         return kmi_set_error(KMI_E_SHAPE, "%s: tiled layout needs N%%%d==0, got N=%d", fn, KMI_TILE_N, N);
     if (M < 0) return kmi_set_error(KMI_E_SHAPE, "%s: need M>=0, got %d", fn, M);
     const long chunks = (long)N * K / 32;
-    const dim3 grid((unsigned)(M + (chunks + 255) / 256));
+    const dim3 grid((unsigned)M + (unsigned)((chunks + 255) / 256));
     const int cpt = ((K >> 3) + 255) / 256;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const u4_t* q = static_cast<const u4_t*>(qweight);
