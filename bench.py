@@ -181,7 +181,6 @@ def main():
     from kairos_amd import ops
     from kairos_amd.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
     from kairos_amd.perf_profiler import Profiler
-    from kairos_amd.weight_prep import prepare_linear_weight
     from oracle import kairos_oracle as O                     # synthetic inputs + the CPU leg only
 
     dev = torch.device("cuda:0")
@@ -191,7 +190,7 @@ def main():
     # ---- synthetic layer copies --------------------------------------------------------------
     layers = []
     for _name, N, K in LAYER:
-        prep = {k: v.to(dev) for k, v in prepare_linear_weight(torch.from_numpy(O.synth_weights(N, K, seed=10))).items()}
+        prep = ops.prepare_weight(torch.from_numpy(O.synth_weights(N, K, seed=10)).to(dev))
         copies = []
         for c in range(args.copies):
             dl = DynamicLinear(K, N, False, dev, 128)

@@ -85,6 +85,24 @@ int kmi_quant_act_i8(void* out_i8, void* scale_f16, const void* x_f16, int M, in
 int kmi_prep_w8a8(void* w8_out, int tiled, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
                   int N, int K, int G, void* a8_out, void* ascale_f16, const void* x_f16, int M, void* stream);
 
+/* ---- offline weight preparation ----------------------------------------------------------------- */
+
+/* fp16 weight [N, K] (row-major) -> the resident format of one linear, in one launch:
+ *   qweight [N/4, K] int16 (four-row interleave, 4 nibbles per word), scales / scaled_zeros [Gp, N] fp16 (W4A16
+ *   lanes), scales_to8 / scaled_zeros_to8 [Gp, N] fp16 (int4 -> int8 conversion), scales_1 [N] fp16 (per channel),
+ *   Gp = kmi_padded_groups(K, G); padded table rows are written as zeros.
+ * Replaces the torch chain of DynamicLinear.from_module (kairos/dynamic_linear.py:86-115): quantize_tensor_int8
+ * (kairos/quantization.py:112-141), kairos_quantize_tensor_int4 (kairos/dynamic_linear_v2.py:15-41), pack_int_awq
+ * and trans_qfactor_layout_awq (thirdparty/AWQ/awq_method.py:5-75), with the same fp32 / fp16 operations in the
+ * same order, so every output equals the host chain bit for bit.  Needs N%4==0, K%128==0, G==128; weights must be
+ * finite. */
+int kmi_prepare_weight(const void* w_f16, int N, int K, int G, void* qweight, void* scales, void* scaled_zeros,
+                       void* scales_to8, void* scaled_zeros_to8, void* scales_1, void* stream);
+
+/* Rows of the scale tables for in_features K: 8 * ceil((K/G) / 8) (calculate_zeros_width,
+ * thirdparty/AWQ/awq_method.py:40-54).  Host only; negative error code for unsupported arguments. */
+int kmi_padded_groups(int K, int G);
+
 /* ---- W4A16, small M ---------------------------------------------------------------------------- */
 
 /* out = x . dequant(qweight)^T (+bias), weights streamed once, fp32 accumulation on MFMA.

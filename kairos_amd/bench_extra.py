@@ -3,6 +3,7 @@
     python -m kairos_amd.bench_extra gemv70b   # decode-regime W4A16 on Llama-3-70B shapes, M = 1..32
     python -m kairos_amd.bench_extra convert   # int4 -> int8 / fp16 / tiled conversion on Qwen2.5-7B shapes
     python -m kairos_amd.bench_extra decoder   # random-init Llama-3-8B decoder: TTFT / TPOT / lane switches
+    python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format, device kernel vs host chain
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -21,7 +22,6 @@ from . import ops
 from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
 from .perf_profiler import Profiler
 from .temp_cache import TempCache
-from .weight_prep import prepare_linear_weight
 
 HBM = 8.0e12
 G = 128
@@ -54,7 +54,7 @@ def _time(fn, n):
 
 def _layer(N, K, copies, dev):
     """One prepared linear, `copies` times in distinct memory (the values do not matter for timing)."""
-    prep = {k: v.to(dev) for k, v in prepare_linear_weight(_weights(min(N, 1024), K)).items()}
+    prep = ops.prepare_weight(_weights(min(N, 1024), K).to(dev))
     reps = N // min(N, 1024)
     full = {"qweight": prep["qweight"].repeat(reps, 1), "scales_1": prep["scales_1"].repeat(reps)}
     for k in ("scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8"):
@@ -120,6 +120,41 @@ def convert(args):
     assert cache.peak_bytes <= largest and cache.capacity <= largest, (cache.peak_bytes, cache.capacity, largest)
     return {"bench": "convert", "rows": rows, "temp_cache_peak_bytes": cache.peak_bytes,
             "largest_converted_weight_bytes": largest, "temp_cache_bounded": True}
+
+
+def weightprep(args):
+    """Offline preparation (DynamicLinear.from_module's chain) on Llama-3-8B and -70B shapes: the device kernel
+    against the HBM roofline (fp16 weight in, packed int4 + four tables + channel scales out), with the host torch
+    chain timed on a 1024-row slice and scaled to the full weight beside it."""
+    from .weight_prep import prepare_linear_weight
+    dev = torch.device("cuda:0")
+    rows = []
+    for name, N, K in [("8b_qkv", 6144, 4096), ("8b_o", 4096, 4096), ("8b_gate_up", 28672, 4096), ("8b_down", 4096, 14336),
+                       ("70b_qkv", 10240, 8192), ("70b_gate_up", 57344, 8192), ("70b_down", 8192, 28672)]:
+        copies = max(2, math.ceil(600e6 / (N * K * 2)))
+        base = _weights(min(N, 1024), K)
+        w = [base.repeat(N // min(N, 1024), 1).to(dev) * (1.0 + 0.01 * c) for c in range(copies)]
+        out = ops.prepare_weight(w[0])
+        lib = ops._lib.load()
+
+        def call(i):
+            ops._lib.check(lib.kmi_prepare_weight(w[i % copies].data_ptr(), N, K, G, out["qweight"].data_ptr(),
+                                                  out["scales"].data_ptr(), out["scaled_zeros"].data_ptr(),
+                                                  out["scales_to8"].data_ptr(), out["scaled_zeros_to8"].data_ptr(),
+                                                  out["scales_1"].data_ptr(), ops._stream()))
+        us = _time(call, 20)
+        b = N * K * 2 + N * K // 2 + 4 * (K // G) * N * 2 + 2 * N
+        t0 = time.perf_counter()
+        prepare_linear_weight(base)
+        host_s = (time.perf_counter() - t0) * (N / base.shape[0])
+        rows.append({"shape": name, "N": N, "K": K, "us": round(us, 1), "gbps": round(b / us / 1e3, 1),
+                     "hbm_frac": round(b / us / 1e-6 / HBM, 4), "host_chain_ms": round(host_s * 1e3, 1),
+                     "host_threads": torch.get_num_threads()})
+        print(rows[-1], file=sys.stderr, flush=True)
+        del w, out
+        torch.cuda.empty_cache()
+    return {"bench": "weightprep", "rows": rows,
+            "algorithmic_bytes": "2*N*K (fp16 in) + N*K/2 (int4 out) + 4*(K/128)*N*2 (tables) + 2*N (channel scales)"}
 
 
 # ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
@@ -240,6 +275,7 @@ def main(argv=None):
     sub = ap.add_subparsers(dest="cmd", required=True)
     sub.add_parser("gemv70b")
     sub.add_parser("convert")
+    sub.add_parser("weightprep")
     d = sub.add_parser("decoder")
     d.add_argument("--lut", default=None)
     d.add_argument("--layers", type=int, default=32)
@@ -254,7 +290,7 @@ def main(argv=None):
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
     ops.ensure_workspace()
-    res = {"gemv70b": gemv70b, "convert": convert, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

@@ -60,10 +60,15 @@ class DynamicLinear(torch.nn.Module):
         q_linear = cls(linear.in_features, linear.out_features, linear.bias is not None, device, group_size=128)
         if init_only:
             return q_linear
-        # Quantisation runs on the host: ROCm PyTorch's elementwise fp32 division is not correctly
-        # rounded, so the same torch ops on the GPU flip round-half-even ties and give a (slightly)
-        # different int4 tensor than the reference arithmetic.  The packed result is then uploaded.
-        prepared = prepare_linear_weight(linear.weight.data.detach().cpu(), group_size=128)
+        # On a GPU the whole chain (int8 per channel -> uint4 per group -> packed words and tables) is one kernel
+        # of the library.  The same torch ops on a ROCm device would not do: PyTorch's elementwise fp32 division
+        # there is not correctly rounded, which flips round-half-even ties against the reference arithmetic.
+        # A CPU target keeps the host chain (weight_prep), which yields the same bits.
+        if torch.device(device).type == 'cuda':
+            w = linear.weight.data.detach().to(device=device, dtype=torch.float16).contiguous()
+            prepared = ops.prepare_weight(w, group_size=128)
+        else:
+            prepared = prepare_linear_weight(linear.weight.data.detach().cpu(), group_size=128)
         for key, value in prepared.items():
             setattr(q_linear, key, value.to(device))
         if linear.bias is not None:

@@ -110,6 +110,30 @@ def prep_w8a8(w8_out, qweight, scale_to8, scaled_zero_to8, int_x, x, scale_x, gr
           x.data_ptr(), M, _stream())
 
 
+def prepare_weight(weight, group_size=GROUP_SIZE):
+    """fp16 [N, K] weight on the GPU -> dict of the six resident tensors (DynamicLinear.from_module,
+    kairos/dynamic_linear.py:95-111), computed by one kernel; bit-identical to weight_prep.prepare_linear_weight."""
+    _need(weight, torch.float16, "weight")
+    if weight.dim() != 2:
+        raise ValueError(f"prepare_weight: weight must be 2-D, got {tuple(weight.shape)}")
+    N, K = weight.shape
+    lib = _lib.load()
+    gp = lib.kmi_padded_groups(K, group_size)
+    if gp < 0:
+        raise ValueError(lib.kmi_get_last_error_string().decode())
+    dev = weight.device
+    out = {"qweight": torch.empty((max(N // 4, 0), K), dtype=torch.int16, device=dev),
+           "scales": torch.empty((gp, N), dtype=torch.float16, device=dev),
+           "scaled_zeros": torch.empty((gp, N), dtype=torch.float16, device=dev),
+           "scales_to8": torch.empty((gp, N), dtype=torch.float16, device=dev),
+           "scaled_zeros_to8": torch.empty((gp, N), dtype=torch.float16, device=dev),
+           "scales_1": torch.empty((N,), dtype=torch.float16, device=dev)}
+    _call("prepare_weight", 0, N, K, lib.kmi_prepare_weight, weight.data_ptr(), N, K, group_size,
+          out["qweight"].data_ptr(), out["scales"].data_ptr(), out["scaled_zeros"].data_ptr(),
+          out["scales_to8"].data_ptr(), out["scaled_zeros_to8"].data_ptr(), out["scales_1"].data_ptr(), _stream())
+    return out
+
+
 # ---- products -----------------------------------------------------------------------------------
 def _flat2d(x):
     return x.reshape(-1, x.shape[-1])

@@ -59,6 +59,15 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_gemm_w4a16_wp_rows(16, 4096, 4096) == 32
     assert lib.kmi_gemm_w4a16_wp_rows(4096, 4096, 4096) == 0
     assert lib.kmi_gemm_pick_tile(4096, 4096) == 256 and lib.kmi_gemm_pick_tile(8, 4096) == 64
+    # offline weight preparation: same shape rules as the converters; table height is host arithmetic
+    assert lib.kmi_prepare_weight(None, 8, 128, 128, 16, 16, 16, 16, 16, 16, None) == -1
+    assert lib.kmi_prepare_weight(16, 6, 128, 128, 16, 16, 16, 16, 16, 16, None) == -2
+    assert lib.kmi_prepare_weight(16, 8, 192, 128, 16, 16, 16, 16, 16, 16, None) == -2
+    assert lib.kmi_prepare_weight(16, 8, 128, 64, 16, 16, 16, 16, 16, 16, None) == -3
+    assert lib.kmi_prepare_weight(8, 8, 128, 128, 16, 16, 16, 16, 16, 16, None) == -5
+    for K in (128, 1024, 3584, 4096, 14336, 18944, 28672):
+        assert lib.kmi_padded_groups(K, 128) == O.padded_groups(K)
+    assert lib.kmi_padded_groups(100, 128) == -2 and lib.kmi_padded_groups(128, 64) == -2
     assert lib.kmi_lut_get(None, 3) == -7
 
 

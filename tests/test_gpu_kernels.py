@@ -469,3 +469,103 @@ def test_gemm_w4a16_variants_agree_at_full_size(ops, M, N, K):
     if M <= 64:
         v = ops.gemv_forward(x, qw, s, z, M, N, K, 128).float()
         assert ((a - v).abs().max() / scale).item() < 2e-3
+
+
+# ------------------------------------------------------------------ offline weight preparation on the device, bit-exact
+PREP_KEYS = ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1")
+
+
+def check_prepare(ops, w):
+    want = O.prepare_weights(w)
+    got = ops.prepare_weight(dev(w))
+    for key in PREP_KEYS:
+        g, r = host(got[key]), want[key]
+        if g.dtype == np.float16:          # 0 * inf in a degenerate group: NaN on both sides, sign and payload are not defined
+            both_nan = np.isnan(g) & np.isnan(r)
+            g, r = np.where(both_nan, np.float16(0), g), np.where(both_nan, np.float16(0), r)
+        assert_same_bits(g, r)
+
+
+@pytest.mark.parametrize("N,K", [(4, 128), (8, 256), (64, 512), (128, 3584), (64, 18944), (256, 4096), (36, 640)])
+def test_prepare_weight_bit_exact(ops, N, K):
+    check_prepare(ops, O.synth_weights(N, K, seed=N + K))
+
+
+def test_prepare_weight_edge_rows(ops):
+    """Rows and groups the arithmetic treats specially: all-zero rows (scale clamps, -0 zero-points), constant groups
+    (zero-point overflows fp16 to -inf as on the host), outliers (most groups collapse to few levels), exact ties."""
+    rng = np.random.default_rng(5)
+    N, K = 32, 1024
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    w[0] = 0
+    w[1, :128] = np.float16(0.0123)
+    w[2] = np.float16(-0.5)
+    w[3, 7] = np.float16(30.0)
+    w[4] = (rng.integers(-127, 128, K) * 0.5).astype(np.float16)          # x/s lands on .5 ties after step 1
+    w[4, 0] = np.float16(63.5)
+    w[5, :] = np.float16(6e-8)                                            # fp16 subnormals
+    w[6, ::2] = np.float16(65504.0)
+    w[7] = np.where(np.arange(K) % 128 < 64, np.float16(1.0), np.float16(-1.0))
+    with np.errstate(over="ignore", invalid="ignore"):
+        check_prepare(ops, w)
+
+
+def test_prepare_weight_feeds_the_kernels(ops):
+    """End to end: device-prepared tensors through the converter equal the oracle's conversion of its own preparation."""
+    N, K = 256, 1024
+    w = O.synth_weights(N, K, seed=3)
+    got = ops.prepare_weight(dev(w))
+    p = prep(N, K, 3)
+    out = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(out, got["qweight"], got["scales_to8"], got["scaled_zeros_to8"], 128)
+    assert_same_bits(host(out), p["w8"])
+
+
+def test_prepare_weight_rejects_bad_arguments(ops):
+    with pytest.raises(TypeError):
+        ops.prepare_weight(torch.zeros((8, 128), device="cuda"))
+    with pytest.raises(Exception):
+        ops.prepare_weight(torch.zeros((6, 128), dtype=torch.float16, device="cuda"))
+    with pytest.raises(Exception):
+        ops.prepare_weight(torch.zeros((8, 192), dtype=torch.float16, device="cuda"))
+
+
+def test_prepare_weight_every_group_range(ops):
+    """Step 2 exhaustively: every reachable (lo, hi, x) of a group of int8 values.  Rows hold integers and a +-127, so
+    step 1 is the identity (s1 = 1); each later group spans one (lo, hi) pair and carries every value between."""
+    groups = []
+    for lo in range(-127, 128):
+        groups.append([lo] * 128)                                             # constant group
+        for hi in range(lo + 1, 128):
+            inner = list(range(lo + 1, hi))
+            for at in range(0, max(len(inner), 1), 126):
+                piece = inner[at:at + 126]
+                groups.append([lo, hi] + piece + [lo] * (126 - len(piece)))
+    per_row = 31
+    rows = -(-len(groups) // per_row)
+    rows += -rows % 4
+    groups += [groups[-1]] * (rows * per_row - len(groups))
+    body = np.asarray(groups, dtype=np.float16).reshape(rows, per_row * 128)
+    first = np.zeros((rows, 128), dtype=np.float16)
+    first[:, 0], first[:, 1] = 127, -127
+    w = np.concatenate([first, body], axis=1)
+    assert w.shape[1] == 4096
+    with np.errstate(over="ignore", invalid="ignore"):
+        check_prepare(ops, w)
+
+
+def test_prepare_weight_every_numerator(ops):
+    """Step 1 for 64 divisors (row maxima, drawn over the whole fp16 range, edge values included): every positive
+    finite fp16 value up to the maximum appears in the row, so each division w / s1 the row can need is checked."""
+    rng = np.random.default_rng(9)
+    allpos = np.arange(1, 0x7C00, dtype=np.uint16).view(np.float16)           # every positive finite fp16, ascending
+    tops = list(rng.integers(1, 0x7C00, 58).astype(np.uint16).view(np.float16))
+    tops += [np.float16(65504), np.float16(1.0), np.float16(127.0), np.float16(6e-8), np.float16(6.1e-5), np.float16(0.02)]
+    K = 32768
+    w = np.zeros((64, K), dtype=np.float16)
+    for i, top in enumerate(tops):
+        vals = allpos[allpos <= top]
+        w[i, :len(vals)] = vals
+        w[i, len(vals):] = -np.resize(vals, K - len(vals))                    # the same values, negative, repeated
+    with np.errstate(over="ignore", invalid="ignore"):
+        check_prepare(ops, w)
