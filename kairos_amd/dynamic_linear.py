@@ -18,19 +18,21 @@ import torch
 
 from . import ops
 from .temp_cache import default_cache
-from .weight_prep import prepare_linear_weight
+from .weight_prep import calculate_zeros_width, prepare_linear_weight
 
 COMP_TYPE_NAME = {'w4a16_gemm': 0, 'w4a16_gemv': 1, 'w8a8': 2,
                   'w8a16_gemm': 3, 'w8a16_gemv': 4, 'fp16': 5}
 
 _W4A16_GEMM, _W4A16_GEMV, _W8A8, _W8A16_GEMM, _W8A16_GEMV, _FP16 = 0, 1, 2, 3, 4, 5
 _uids = itertools.count(1)
+RESIDENT_KEYS = ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1")
 
 
 class DynamicLinear(torch.nn.Module):
     prof = None                 # Profiler shared by every instance, set by the caller (kairos/main.py:52)
     tiled_weights = True        # converted weights are written in the tiled MFMA staging layout
     temp_cache = None           # None -> the process-wide default cache
+    resident_copies = False     # True (SwitchLinear): converted weights are kept per layer, no lane converts
 
     @torch.no_grad()
     def __init__(self, in_features, out_features, bias, device, group_size):
@@ -51,14 +53,48 @@ class DynamicLinear(torch.nn.Module):
         self._uid = next(_uids)     # identifies this layer's entries in the temp cache
         self._decode_ptrs = None
         self.switch_count = 0       # times the selected lane changed between consecutive forward calls
-        self.qweight = self.scales = self.scaled_zeros = None
-        self.scales_to8 = self.scaled_zeros_to8 = self.scales_1 = None
+        # The six resident tensors are buffers, so state_dict() / load_state_dict() carry the quantised layer
+        # (the reference keeps them as plain attributes, which torch.save(model.state_dict()) silently drops,
+        # kairos/main.py:85-91).  None until from_module fills or allocates them.
+        for key in RESIDENT_KEYS:
+            self.register_buffer(key, None)
+
+    def _allocate_resident(self, device):
+        """Uninitialised resident tensors of the right shapes: the target of load_state_dict (init_only modules)."""
+        N, K = self.shape
+        gp = calculate_zeros_width(K, self.group_size) * 8
+        self.qweight = torch.empty((N // 4, K), dtype=torch.int16, device=device)
+        for key in ("scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8"):
+            setattr(self, key, torch.empty((gp, N), dtype=torch.float16, device=device))
+        self.scales_1 = torch.empty((N,), dtype=torch.float16, device=device)
+
+    def init(self):
+        """After the resident tensors changed in place or moved (load_state_dict, .to()): forget everything derived
+        from the old ones -- cached pointers, the lane memo and this layer's entries in the temp cache
+        (kairos/dynamic_linear.py:81-83 is the reference's hook of the same name)."""
+        self._decode_ptrs = None
+        self.pre_m = 0
+        self.comp_type = None
+        self._uid = next(_uids)
+
+    def _apply(self, fn, *args, **kwargs):
+        out = super()._apply(fn, *args, **kwargs)
+        self.init()
+        return out
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        if self.qweight is None and prefix + "qweight" in state_dict:      # plain constructor: allocate on the fly
+            dev = state_dict[prefix + "qweight"].device if self.bias is None else self.bias.device
+            self._allocate_resident(dev)
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+        self.init()
 
     @classmethod
     @torch.no_grad()
     def from_module(cls, linear, device, return_dtype=torch.float16, init_only=False, name=''):
         q_linear = cls(linear.in_features, linear.out_features, linear.bias is not None, device, group_size=128)
         if init_only:
+            q_linear._allocate_resident(device)
             return q_linear
         # On a GPU the whole chain (int8 per channel -> uint4 per group -> packed words and tables) is one kernel
         # of the library.  The same torch ops on a ROCm device would not do: PyTorch's elementwise fp32 division
@@ -144,8 +180,11 @@ class DynamicLinear(torch.nn.Module):
         elif comp_type == _W8A8:
             int_x = torch.empty_like(x, dtype=torch.int8)
             scale_x = torch.empty((m,), device=x.device, dtype=torch.float16)
-            tiled = self._tileable()
-            w8, hit = self._cache().get(self._uid, ('i8', tiled), self.shape, torch.int8, self.qweight.device)
+            if self.resident_copies:
+                (w8, tiled), hit = self._converted('i8'), True
+            else:
+                tiled = self._tileable()
+                w8, hit = self._cache().get(self._uid, ('i8', tiled), self.shape, torch.int8, self.qweight.device)
             if hit:
                 ops.quant_fp16_to_int8(int_x, x, scale_x)
             else:                                            # conversion and quantisation share one launch

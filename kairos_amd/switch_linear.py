@@ -12,25 +12,45 @@ from .dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear
 
 class SwitchLinear(DynamicLinear):
     prof = None
+    resident_copies = True
+
+    def init(self):
+        super().init()
+        self._resident = None           # (int8 weight, fp16 weight, int8 row-major or None, tiled), built on first use
+
+    def _ensure_resident(self):
+        """The int8 and fp16 copies are derived data: not part of state_dict, rebuilt after a load or a move."""
+        if getattr(self, "_resident", None) is None:
+            dev, tiled = self.qweight.device, self._tileable()
+            w8 = torch.empty(self.shape, dtype=torch.int8, device=dev)
+            ops.dequant_interleaved_int4_to_int8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8, 128, tiled=tiled)
+            w16 = torch.empty(self.shape, dtype=torch.float16, device=dev)
+            ops.dequant_interleaved_int4_to_fp16(w16, self.qweight, self.scales, self.scaled_zeros, 128, tiled=tiled)
+            w8_rows = None
+            if tiled:       # the W8A16 lane reads row-major int8
+                w8_rows = torch.empty(self.shape, dtype=torch.int8, device=dev)
+                ops.dequant_interleaved_int4_to_int8(w8_rows, self.qweight, self.scales_to8, self.scaled_zeros_to8, 128)
+            self._resident = (w8, w16, w8_rows, tiled)
+        return self._resident
+
+    @property
+    def smq_weight(self):               # names of the reference's attributes (kairos/switch_linear.py:43-213)
+        return self._ensure_resident()[0]
+
+    @property
+    def ori_weight(self):
+        return self._ensure_resident()[1]
 
     @classmethod
     @torch.no_grad()
     def from_module(cls, linear, device, return_dtype=torch.float16, init_only=False, name=''):
         q = super().from_module(linear, device, return_dtype, init_only, name)
-        if init_only:
-            return q
-        tiled = q._tileable()
-        q.smq_weight = torch.empty(q.shape, dtype=torch.int8, device=device)
-        ops.dequant_interleaved_int4_to_int8(q.smq_weight, q.qweight, q.scales_to8, q.scaled_zeros_to8, 128, tiled=tiled)
-        q.ori_weight = torch.empty(q.shape, dtype=torch.float16, device=device)
-        ops.dequant_interleaved_int4_to_fp16(q.ori_weight, q.qweight, q.scales, q.scaled_zeros, 128, tiled=tiled)
-        q._resident_tiled = tiled
-        if tiled:       # the W8A16 lane reads row-major int8
-            q.smq_weight_rowmajor = torch.empty(q.shape, dtype=torch.int8, device=device)
-            ops.dequant_interleaved_int4_to_int8(q.smq_weight_rowmajor, q.qweight, q.scales_to8, q.scaled_zeros_to8, 128)
+        if not init_only and torch.device(device).type == 'cuda':
+            q._ensure_resident()
         return q
 
     def _converted(self, fmt, tiled=None):
-        if fmt == 'i8' and tiled is False and self._resident_tiled:
-            return self.smq_weight_rowmajor, False
-        return (self.smq_weight if fmt == 'i8' else self.ori_weight), self._resident_tiled
+        w8, w16, w8_rows, res_tiled = self._ensure_resident()
+        if fmt == 'i8' and tiled is False and res_tiled:
+            return w8_rows, False
+        return (w8 if fmt == 'i8' else w16), res_tiled

@@ -161,3 +161,34 @@ def test_graph_replay_matches_eager():
         assert g.replays == 12
     finally:
         DynamicLinear.prof = old
+
+
+@pytest.mark.parametrize("cls_name", ["DynamicLinear", "SwitchLinear"])
+def test_checkpoint_round_trip_keeps_every_lane(gpu, cls_name, tmp_path):
+    """Dump a quantised layer, load it into an init_only module (on the CPU, then moved to the GPU, as
+    utils/load_model.py:15-29 does) and into a live module that holds other weights: every lane returns the bits of
+    the original, and nothing derived from the replaced weights (temp-cache entries, resident copies) survives."""
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos.switch_linear import SwitchLinear
+    cls = {"DynamicLinear": DynamicLinear, "SwitchLinear": SwitchLinear}[cls_name]
+    N, K = 256, 1024
+    lin, _ = make_linear(N, K, True, seed=21)
+    src = cls.from_module(lin.cuda(), 'cuda')
+    xs = {M: torch.from_numpy(O.synth_acts(M, K, seed=M)).cuda()[None] for M in (3, 70, 300)}
+    want = {(M, cid): src._forward(x, M, cid).clone() for M, x in xs.items() for cid in COMP_TYPE_NAME.values()}
+    path = tmp_path / "layer.pt"
+    torch.save(src.state_dict(), path)
+
+    fresh = cls.from_module(lin, 'cpu', init_only=True)
+    fresh.load_state_dict(torch.load(path, weights_only=True))
+    fresh = fresh.cuda()
+    other, _ = make_linear(N, K, True, seed=22)
+    live = cls.from_module(other.cuda(), 'cuda')
+    for M, x in xs.items():                                  # fill caches / resident copies with the OTHER weights
+        live._forward(x, M, COMP_TYPE_NAME['w8a8'])
+        live._forward(x, M, COMP_TYPE_NAME['fp16'])
+    live.load_state_dict(torch.load(path, weights_only=True))
+    for mod in (fresh, live):
+        for (M, cid), ref in want.items():
+            out = mod._forward(xs[M], M, cid)
+            assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (cls_name, M, cid)

@@ -92,10 +92,39 @@ def test_from_module_on_cpu_matches_oracle_and_refuses_cpu_compute():
     assert dl.shape == (64, 256) and dl.pre_m == 0 and dl.group_size == 128
     assert torch.equal(dl.bias, lin.bias.detach())
     assert "in_features=256, out_features=64, bias=True" in repr(dl)
-    empty = DynamicLinear.from_module(lin, 'cpu', init_only=True)
-    assert empty.qweight is None
+    assert DynamicLinear(256, 64, False, 'cpu', 128).qweight is None     # the plain constructor allocates nothing
     with pytest.raises((ValueError, ImportError)):      # no CPU fallback: the HIP path is the only path
         dl._forward(torch.zeros(1, 2, 256, dtype=torch.float16), 2, 1)
+
+
+def test_state_dict_round_trip_on_cpu(tmp_path):
+    """The six resident tensors (and the bias) travel through state_dict / torch.save / load_state_dict; an
+    init_only module has the right shapes to receive them (kairos/main.py:85-91, utils/load_model.py:15-29)."""
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos_amd.dynamic_linear import RESIDENT_KEYS
+    torch.manual_seed(1)
+    model = torch.nn.Sequential(torch.nn.Linear(256, 64, bias=True, dtype=torch.float16),
+                                torch.nn.Linear(128, 64, bias=False, dtype=torch.float16))
+    q = torch.nn.Sequential(*[DynamicLinear.from_module(l, 'cpu') for l in model])
+    sd = q.state_dict()
+    assert set(sd) == {f"{i}.{k}" for i in (0, 1) for k in RESIDENT_KEYS} | {"0.bias"}
+    path = tmp_path / "q_model.pt"
+    torch.save(sd, path)
+    loaded = torch.load(path, weights_only=True)
+    fresh = torch.nn.Sequential(*[DynamicLinear.from_module(l, 'cpu', init_only=True) for l in model])
+    assert fresh[0].qweight.shape == (16, 256) and fresh[1].scales.shape == (8, 64)
+    uid = fresh[0]._uid
+    fresh.load_state_dict(loaded)                       # strict
+    assert fresh[0]._uid != uid                         # stale temp-cache entries of this layer can no longer hit
+    for a, b in zip(q, fresh):
+        for k in RESIDENT_KEYS:
+            assert torch.equal(getattr(a, k), getattr(b, k)) and getattr(a, k).dtype == getattr(b, k).dtype, k
+    assert torch.equal(q[0].bias, fresh[0].bias)
+    bare = DynamicLinear(128, 64, False, 'cpu', 128)    # plain constructor: allocated while loading
+    bare.load_state_dict({k: getattr(q[1], k) for k in RESIDENT_KEYS})
+    assert torch.equal(bare.qweight, q[1].qweight)
+    with pytest.raises(RuntimeError):                   # a checkpoint of another shape is refused
+        fresh[0].load_state_dict(q[1].state_dict())
 
 
 def test_temp_cache_is_bounded_and_reuses():
