@@ -103,6 +103,15 @@ int kmi_prepare_weight(const void* w_f16, int N, int K, int G, void* qweight, vo
  * thirdparty/AWQ/awq_method.py:40-54).  Host only; negative error code for unsupported arguments. */
 int kmi_padded_groups(int K, int G);
 
+/* ---- re-pack for the version-2 W4A8 candidate --------------------------------------------------- */
+
+/* Resident packed int4 [N/4, K] -> int8 [N, K/2] in the W4A8 operand layout (32x32 blocks of 512 bytes; byte
+ * (n%8)*64 + ((k%16)/4)*16 + ((k%32)/16)*8 + ((n%16)/8)*4 + k%4 of block (n/32, k/32) holds row n in the low and
+ * row n+16 in the high nibble).  Replaces trans_layout_c16_to_c8_awq (kernels/csrc/pybind.cpp:24,
+ * kernels/csrc/kairos_kernel/trans_layout/trans_layout_marlin_c16_to_c8.cu:183-205); bit-exact contract
+ * test/test_trans_layout.py:46-52.  Needs N%32==0, K%64==0. */
+int kmi_trans_layout_w4a8(void* out_i8, const void* qweight, int N, int K, void* stream);
+
 /* ---- W4A16, small M ---------------------------------------------------------------------------- */
 
 /* out = x . dequant(qweight)^T (+bias), weights streamed once, fp32 accumulation on MFMA.

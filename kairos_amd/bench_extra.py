@@ -3,7 +3,7 @@
     python -m kairos_amd.bench_extra gemv70b   # decode-regime W4A16 on Llama-3-70B shapes, M = 1..32
     python -m kairos_amd.bench_extra convert   # int4 -> int8 / fp16 / tiled conversion on Qwen2.5-7B shapes
     python -m kairos_amd.bench_extra decoder   # random-init Llama-3-8B decoder: TTFT / TPOT / lane switches
-    python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format, device kernel vs host chain
+    python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -150,8 +150,12 @@ def weightprep(args):
         rows.append({"shape": name, "N": N, "K": K, "us": round(us, 1), "gbps": round(b / us / 1e3, 1),
                      "hbm_frac": round(b / us / 1e-6 / HBM, 4), "host_chain_ms": round(host_s * 1e3, 1),
                      "host_threads": torch.get_num_threads()})
+        # re-pack of the resident format into the W4A8 operand layout (pure nibble shuffle: N*K/2 in, N*K/2 out)
+        packs = [torch.randint(-32768, 32767, (N // 4, K), dtype=torch.int16, device=dev) for _ in range(max(2, copies))]
+        us_r = _time(lambda i: ops.trans_layout_c16_to_c8_awq(packs[i % len(packs)], N, K), 20)
+        rows[-1].update({"repack_us": round(us_r, 1), "repack_hbm_frac": round(N * K / us_r / 1e-6 / HBM, 4)})
         print(rows[-1], file=sys.stderr, flush=True)
-        del w, out
+        del w, out, packs
         torch.cuda.empty_cache()
     return {"bench": "weightprep", "rows": rows,
             "algorithmic_bytes": "2*N*K (fp16 in) + N*K/2 (int4 out) + 4*(K/128)*N*2 (tables) + 2*N (channel scales)"}

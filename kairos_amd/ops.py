@@ -134,6 +134,18 @@ def prepare_weight(weight, group_size=GROUP_SIZE):
     return out
 
 
+def trans_layout_c16_to_c8_awq(awq_packed, N, K):
+    """Resident packed int4 [N/4, K] -> int8 [N, K/2] in the W4A8 operand layout; allocates and returns the output
+    as the reference binding does (trans_layout_marlin_c16_to_c8.cu:183-205)."""
+    _need(awq_packed, torch.int16, "awq_packed")
+    if awq_packed.numel() != (N // 4) * K:
+        raise ValueError(f"trans_layout_c16_to_c8_awq: tensor of {awq_packed.numel()} words does not match N={N} K={K}")
+    out = torch.empty((N, K // 2), dtype=torch.int8, device=awq_packed.device)
+    _call("trans_layout_w4a8", 0, N, K, _lib.load().kmi_trans_layout_w4a8, out.data_ptr(), awq_packed.data_ptr(), N, K,
+          _stream())
+    return out
+
+
 # ---- products -----------------------------------------------------------------------------------
 def _flat2d(x):
     return x.reshape(-1, x.shape[-1])

@@ -25,6 +25,11 @@ Pinning status (what, other than this file agreeing with itself, fixes each func
                                   accumulated matmul, tolerance 1e-2 max-abs-rel.
   gemm_w8a16                      parity unpinned: the reference declares the id but has no
                                   implementation (kairos/dynamic_linear.py:8-9).
+  pack_int_w4a8 / trans_layout_   the reference states the layout twice (test/test_trans_layout.py:8-14 in one
+  c16_to_c8                       permutation, thirdparty/Qserve/w4a8_linear.py:187-205 in two) and its own test
+                                  demands trans(pack_awq(A)) == pack_w4a8(A) bit for bit (test_trans_layout.py:46-52);
+                                  both statements re-typed in tests/test_oracle_layout.py plus the index formula
+                                  by brute force.
   LUT                             reference C++ header compiled into oracle/_ref (see Makefile) and
                                   the two shipped table files.
 """
@@ -104,6 +109,50 @@ def unpack_int_awq_by_index(packed):
     nn, kk = np.meshgrid(np.arange(N4 * 4), np.arange(K), indexing="ij")
     word, nib = awq_position(nn, kk, K)
     return ((flat[word] >> (4 * nib).astype(np.uint16)) & 0xF).astype(np.uint8)
+
+
+# ----------------------------------------------------------------------------------------------
+# W4A8 operand layout of the v2 candidate and the re-pack into it      test/test_trans_layout.py:8-52
+# ----------------------------------------------------------------------------------------------
+def w4a8_position(n, k, K):
+    """(flat byte index, nibble) of element (n, k) in the [N, K/2] int8 W4A8 operand.
+
+    32x32 blocks of 512 bytes, block order (n/32, k/32).  Inside a block the byte index is
+    (n%8)*64 + ((k%16)//4)*16 + ((k%32)//16)*8 + ((n%16)//8)*4 + k%4, and rows n and n+16 of the block share a
+    byte: low nibble (n%32) < 16, high nibble otherwise.
+    """
+    n = np.asarray(n, dtype=np.int64)
+    k = np.asarray(k, dtype=np.int64)
+    block = (n // 32) * (K // 32) + k // 32
+    byte = block * 512 + (n % 8) * 64 + ((k % 16) // 4) * 16 + ((k % 32) // 16) * 8 + ((n % 16) // 8) * 4 + k % 4
+    return byte, (n % 32) // 16
+
+
+def pack_int_w4a8(q):
+    """uint4 [N, K] -> int8 [N, K/2] (pack_int_qserve, test/test_trans_layout.py:8-14)."""
+    q = np.asarray(q)
+    N, K = q.shape
+    assert N % 32 == 0 and K % 32 == 0
+    v = (q.astype(np.uint8) & 0xF).reshape(N // 32, 2, 2, 8, K // 32, 2, 4, 4)
+    v = v.transpose(0, 4, 3, 6, 5, 2, 7, 1)
+    return np.ascontiguousarray((v[..., 1] << 4) + v[..., 0]).reshape(N, K // 2).view(np.int8)
+
+
+def pack_int_w4a8_by_index(q):
+    q = np.asarray(q)
+    N, K = q.shape
+    nn, kk = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
+    byte, nib = w4a8_position(nn, kk, K)
+    out = np.zeros(N * K // 2, dtype=np.uint8)
+    np.bitwise_or.at(out, byte.ravel(), ((q.astype(np.uint8) & 0xF) << (4 * nib).astype(np.uint8)).ravel())
+    return out.view(np.int8).reshape(N, K // 2)
+
+
+def trans_layout_c16_to_c8(packed):
+    """Resident packed int4 [N/4, K] -> W4A8 operand [N, K/2]: the same nibbles, re-ordered
+    (trans_layout_c16_to_c8_awq, kernels/csrc/kairos_kernel/trans_layout/trans_layout_marlin_c16_to_c8.cu:183-205;
+    contract: test/test_trans_layout.py:46-52)."""
+    return pack_int_w4a8(unpack_int_awq(packed))
 
 
 # ----------------------------------------------------------------------------------------------

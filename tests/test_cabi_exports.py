@@ -68,6 +68,9 @@ def test_argument_validation_needs_no_gpu(lib):
     for K in (128, 1024, 3584, 4096, 14336, 18944, 28672):
         assert lib.kmi_padded_groups(K, 128) == O.padded_groups(K)
     assert lib.kmi_padded_groups(100, 128) == -2 and lib.kmi_padded_groups(128, 64) == -2
+    assert lib.kmi_trans_layout_w4a8(None, 16, 32, 64, None) == -1
+    assert lib.kmi_trans_layout_w4a8(16, 16, 16, 64, None) == -2 and lib.kmi_trans_layout_w4a8(16, 16, 32, 32, None) == -2
+    assert lib.kmi_trans_layout_w4a8(16, 8, 32, 64, None) == -5
     assert lib.kmi_lut_get(None, 3) == -7
 
 

@@ -569,3 +569,22 @@ def test_prepare_weight_every_numerator(ops):
         w[i, len(vals):] = -np.resize(vals, K - len(vals))                    # the same values, negative, repeated
     with np.errstate(over="ignore", invalid="ignore"):
         check_prepare(ops, w)
+
+
+# ------------------------------------------------------------------ re-pack into the W4A8 operand layout, bit-exact
+@pytest.mark.parametrize("N,K", [(32, 64), (64, 192), (96, 3584), (1024, 4096), (4096, 4096), (4096, 14336), (14336, 4096)])
+def test_trans_layout_w4a8_known_answer(ops, N, K):
+    """The reference's own test (test/test_trans_layout.py:46-52, same four large shapes): re-packing the resident
+    format of a random uint4 matrix must equal packing that matrix directly."""
+    q = np.random.default_rng(N ^ K).integers(0, 16, size=(N, K), dtype=np.uint8)
+    got = ops.trans_layout_c16_to_c8_awq(dev(O.pack_int_awq(q)), N, K)
+    assert got.dtype == torch.int8 and tuple(got.shape) == (N, K // 2)
+    assert_same_bits(host(got), O.pack_int_w4a8(q))
+
+
+def test_trans_layout_w4a8_rejects_bad_shapes(ops):
+    t = torch.zeros((8, 64), dtype=torch.int16, device="cuda")
+    with pytest.raises(Exception):
+        ops.trans_layout_c16_to_c8_awq(t, 16, 128)          # N % 32
+    with pytest.raises(ValueError):
+        ops.trans_layout_c16_to_c8_awq(t, 64, 64)           # size mismatch

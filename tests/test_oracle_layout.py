@@ -120,3 +120,59 @@ def test_qfactor_layout_values():
     # hand case: s=0.5, z=3 -> -1.5 exactly
     st, szt = O.qfactor_layout(np.full((4, 1), 0.5, np.float16), np.full((4, 1), 3, np.float16))
     assert (szt[0] == np.float16(-1.5)).all()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# W4A8 operand layout (the v2 candidate's weight format) and the re-pack of the resident format into it.
+# The reference states the layout twice and its own test fixes the re-pack bit for bit:
+#   trans_layout_c16_to_c8_awq(pack_int_awq(A)) == pack_int_qserve(A)          (test/test_trans_layout.py:46-52)
+# ---------------------------------------------------------------------------------------------------------
+def w4a8_one_permutation(q):
+    """test/test_trans_layout.py:8-14."""
+    N, K = q.shape
+    p = q.reshape(N // 32, 2, 2, 8, K // 32, 2, 4, 4).transpose(0, 4, 3, 6, 5, 2, 7, 1)
+    p = np.ascontiguousarray(p).astype(np.int8)
+    return ((p[..., 1] << 4) + p[..., 0]).reshape(N, K // 2)
+
+
+def w4a8_two_permutations(q):
+    """thirdparty/Qserve/w4a8_linear.py:187-205."""
+    N, K = q.shape
+    p = np.ascontiguousarray(q.reshape(N // 32, 2, 2, 8, K // 32, 2, 4, 4).transpose(0, 4, 3, 6, 1, 5, 2, 7))
+    p = np.ascontiguousarray(p.transpose(0, 1, 2, 3, 5, 6, 7, 4)).astype(np.int8)
+    p = (p[..., 1] << 4) + p[..., 0]
+    return p.reshape(N // 32, K // 32, 32, 16).reshape(N, K // 2)
+
+
+def trans_layout_reference_python(awq_packed, N, K):
+    """trans_layout_pytorch, test/test_trans_layout.py:25-37 (the reference's own torch restatement of its kernel)."""
+    a = awq_packed.view(np.uint16).reshape(N // 4, K // 64, 4, 2, 4, 2)
+    u = np.stack([a & 0xF, (a >> 4) & 0xF, (a >> 8) & 0xF, (a >> 12) & 0xF], axis=-1).astype(np.int8)
+    u = u.transpose(0, 2, 1, 3, 6, 4, 5).reshape(N // 32, 2, 2, 8, K // 32, 2, 4, 4)
+    u = u.transpose(0, 4, 3, 6, 5, 2, 7, 1)
+    return np.ascontiguousarray((u[..., 1] << 4) + u[..., 0]).reshape(N, K // 2)
+
+
+@pytest.mark.parametrize("N,K", [(32, 64), (64, 128), (96, 320), (128, 3584)])
+def test_w4a8_layout_statements_agree(N, K):
+    rng = np.random.default_rng(N + K)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    a = O.pack_int_w4a8(q)
+    assert a.dtype == np.int8 and a.shape == (N, K // 2)
+    assert np.array_equal(a, w4a8_one_permutation(q))
+    assert np.array_equal(a, w4a8_two_permutations(q))
+    assert np.array_equal(a, O.pack_int_w4a8_by_index(q))
+    awq = O.pack_int_awq(q)
+    assert np.array_equal(O.trans_layout_c16_to_c8(awq), a)                       # the reference test's contract
+    assert np.array_equal(trans_layout_reference_python(awq, N, K), a)
+
+
+def test_w4a8_layout_brute_force():
+    N, K = 32, 64
+    for n in range(N):
+        for k in range(K):
+            q = np.zeros((N, K), dtype=np.uint8)
+            q[n, k] = 0xF
+            out = O.pack_int_w4a8(q).view(np.uint8).ravel()
+            byte, nib = O.w4a8_position(n, k, K)
+            assert out[byte] == 0xF << (4 * int(nib)) and np.count_nonzero(out) == 1
