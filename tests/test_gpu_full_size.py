@@ -1,0 +1,147 @@
+"""GPU parity at the benchmark's full sizes, where the oracle is too slow to produce every element.
+
+Each test combines (a) whole-matrix properties that any wrong element breaks -- row and column checksums of exact
+integer results against the same sums computed from the inputs (a checksum of checksums), periodicity of the output
+under replicated weights, agreement of independent layouts -- with (b) the oracle on a sample of rows, which are
+independent of each other in every kernel of the path.  Inputs are chosen so that the compared quantities are exactly
+computable (also through the fp16 epilogue), hence the comparisons are bit-exact.
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from oracle import kairos_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from kairos_amd import ops as _ops
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def sample_rows(M, n, seed):
+    rows = np.unique(np.concatenate([[0, M - 1, M // 2, 255, 256], np.random.default_rng(seed).integers(0, M, n)]))
+    return rows[rows < M]
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 28672, 4096), (4096, 4096, 14336), (4096, 6144, 4096)])
+def test_w8a8_accumulators_full_size(ops, M, N, K):
+    """int32 accumulators over full-range int8 operands: both checksums of the whole M x N result and sampled rows."""
+    rng = np.random.default_rng(M + N + K)
+    a8 = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w8 = rng.integers(-128, 128, size=(N, K), dtype=np.int8)
+    acc = ops.w8a8_gemm_acc_i32(dev(a8), dev(w8), N)
+    torch.cuda.synchronize()
+    a64, w64 = a8.astype(np.float64), w8.astype(np.float64)                   # all sums below stay under 2^53: exact
+    row_sum = a64 @ w64.sum(axis=0)                                           # sum_n acc[m, n]
+    col_sum = w64 @ a64.sum(axis=0)                                           # sum_m acc[m, n]
+    assert np.array_equal(acc.sum(dim=1, dtype=torch.int64).cpu().numpy(), row_sum.astype(np.int64))
+    assert np.array_equal(acc.sum(dim=0, dtype=torch.int64).cpu().numpy(), col_sum.astype(np.int64))
+    rows = sample_rows(M, 24, N)
+    assert np.array_equal(acc[torch.from_numpy(rows).cuda()].cpu().numpy(), O.gemm_i8_acc(a8[rows], w8))
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 28672, 4096), (2048, 4096, 14336), (1024, 6144, 4096), (512, 28672, 4096)])
+def test_w8a8_lane_full_size_through_tiled_weights(ops, M, N, K):
+    """The production order of the W8A8 lane at full size: fused preparation launch (int4 -> tiled int8 + activation
+    quantiser), tiled int8 MFMA GEMM (256-row tiles, tail launch where the shape has one), fp16 epilogue.  Tables
+    s = 1, z = -8 make the converted weight the integer q - 8; activations are sparse +-127, so their scale is exactly
+    1 and the quantised row is the row itself; with the channel scale 1/128 the epilogue's fp32 value is exact, so the
+    fp16 output is one known rounding of an exactly computable number: compared bit for bit over the whole matrix."""
+    rng = np.random.default_rng(N + K)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    w8 = q.astype(np.int8) - 8
+    Gp = O.padded_groups(K)
+    ones = torch.ones((Gp, N), dtype=torch.float16, device="cuda")
+    a = np.zeros((M, K), dtype=np.int8)
+    for m in range(M):                                                        # 16 entries of +-1 per row, scaled to +-127 below
+        idx = rng.choice(K, size=16, replace=False)
+        a[m, idx] = rng.choice(np.array([-1, 1], dtype=np.int8), size=16)
+    x = dev((a.astype(np.float16) * np.float16(127.0)))                       # amax = 127 -> scale 1, a8 = +-127
+    w8_t = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    a8 = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    sx = torch.empty((M,), dtype=torch.float16, device="cuda")
+    ops.prep_w8a8(w8_t, dev(O.pack_int_awq(q)), ones, ones * -8.0, a8, x, sx, 128, tiled=True)
+    assert torch.equal(a8.cpu(), torch.from_numpy(a) * 127) and bool((sx == 1.0).all())
+    assert torch.equal(ops.untile(w8_t, N, K).cpu(), torch.from_numpy(w8))    # the tiled converter at full size
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ws = torch.full((N,), 1.0 / 128.0, dtype=torch.float16, device="cuda")    # a power of two: the scaling is exact
+    ops.w8a8_gemm_forward(a8, w8_t, ws, sx, out, tiled=True)
+    torch.cuda.synchronize()
+    # acc = 127 * (a . w8) with |a . w8| <= 16 * 8; out = fp16(fp32(acc) * (1/128 * 1))
+    exact = (a.astype(np.float32) @ w8.astype(np.float32).T) * np.float32(127.0 / 128.0)   # every step exact in fp32
+    want = exact.astype(np.float16)                                           # the one rounding of the epilogue
+    rows = sample_rows(M, 24, K)
+    assert np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy().view(np.uint16), want[rows].view(np.uint16))
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("N,K", [(57344, 8192), (8192, 28672), (10240, 8192)])
+def test_gemv_periodic_weights_70b_shapes(ops, N, K):
+    """Small-M W4A16 at the Llama-3-70B shapes: the weight is a prepared 1024-row slice repeated along N, so every
+    output column must equal, bit for bit, the column 1024 to its left, and the first 1024 columns must match the oracle."""
+    base = 1024
+    p = O.prepare_weights(O.synth_weights(base, K, seed=K))
+    reps = N // base
+    qw = dev(p["qweight"]).repeat(reps, 1)
+    s, z = dev(p["scales"]).repeat(1, reps), dev(p["scaled_zeros"]).repeat(1, reps)
+    for M in (1, 8, 32):
+        x = O.synth_acts(M, K, seed=M)
+        out = ops.gemv_forward(dev(x), qw, s, z, M, N, K, 128)
+        torch.cuda.synchronize()
+        first = out[:, :base]
+        assert torch.equal(out.view(M, reps, base).view(torch.int16), first.view(torch.int16)[:, None, :].expand(M, reps, base))
+        ref = O.gemm_w4a16(x, p["qweight"], p["scales"], p["scaled_zeros"])
+        assert O.max_abs_rel(first.cpu().numpy(), ref) < 1e-2
+
+
+@pytest.mark.parametrize("N,K", [(28672, 4096), (4096, 14336), (37888, 3584)])
+def test_conversion_layouts_agree_full_size(ops, N, K):
+    """Conversion at full size: with s = 1, z = 0 the fp16 result is the unpacked nibble itself (pure layout), the int8
+    result likewise; row-major and tiled outputs must hold the same matrix."""
+    q = np.random.default_rng(N).integers(0, 16, size=(N, K), dtype=np.uint8)
+    qw = dev(O.pack_int_awq(q))
+    Gp = O.padded_groups(K)
+    one = torch.ones((Gp, N), dtype=torch.float16, device="cuda")
+    zero = torch.zeros((Gp, N), dtype=torch.float16, device="cuda")
+    want = torch.from_numpy(q).cuda()
+    for dtype, fn in ((torch.float16, ops.dequant_interleaved_int4_to_fp16), (torch.int8, ops.dequant_interleaved_int4_to_int8)):
+        rows = torch.empty((N, K), dtype=dtype, device="cuda")
+        fn(rows, qw, one, zero, 128)
+        assert torch.equal(rows.to(torch.uint8), want) and bool((rows >= 0).all())
+        if N % 128 == 0:
+            tiled = torch.empty((N, K), dtype=dtype, device="cuda")
+            fn(tiled, qw, one, zero, 128, tiled=True)
+            assert torch.equal(ops.untile(tiled, N, K), rows)
+
+
+def test_module_forward_full_size_rows(ops):
+    """DynamicLinear.forward at M = 4096 on a 4096 x 4096 layer through the W8A8 lane (bit-exact on sampled tokens:
+    every token is quantised and scaled on its own) and at M = 16 through the small-M lane (1e-2)."""
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    N = K = 4096
+    w = O.synth_weights(N, K, seed=10)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16)
+    with torch.no_grad():
+        lin.weight.copy_(torch.from_numpy(w))
+    dl = DynamicLinear.from_module(lin.cuda(), 'cuda')
+    p = O.prepare_weights(w)
+    for key in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1"):
+        assert np.array_equal(getattr(dl, key).cpu().numpy().view(np.uint16), p[key].view(np.uint16)), key
+    M = 4096
+    x = O.synth_acts(M, K, seed=11)
+    out = dl._forward(dev(x)[None], M, COMP_TYPE_NAME['w8a8'])[0]
+    rows = sample_rows(M, 12, 3)
+    ref = O.switched_forward(x[rows], p, COMP_TYPE_NAME['w8a8'])
+    assert np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy().view(np.uint16), ref.view(np.uint16))
+    x16 = O.synth_acts(16, K, seed=12)
+    out16 = dl._forward(dev(x16)[None], 16, COMP_TYPE_NAME['w4a16_gemv'])[0]
+    assert O.max_abs_rel(out16.cpu().numpy(), O.switched_forward(x16, p, COMP_TYPE_NAME['w4a16_gemv'])) < 1e-2
