@@ -164,6 +164,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the small-M layers")
     ap.add_argument("--dump-launches", default=None, help="write every event-bracketed launch of the replay (JSON)")
+    ap.add_argument("--resident-cache-mb", type=int, default=0,
+                    help="keep converted weights in an LRU cache of this many MiB (0 = the single shared temp buffer, "
+                         "which is what the headline figure uses)")
     ap.add_argument("--lut", default=None, help="directory holding seg_perf_list.pt (default: the committed MI355X table)")
     ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -186,6 +189,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     names = {v: k for k, v in COMP_TYPE_NAME.items()}
+
+    if args.resident_cache_mb > 0:
+        from kairos_amd.temp_cache import ResidentCache, set_default_cache
+        set_default_cache(ResidentCache(args.resident_cache_mb << 20))
 
     # ---- synthetic layer copies --------------------------------------------------------------
     layers = []
@@ -385,6 +392,8 @@ def main():
         "config": {"workload": "configs[1]: Llama-3-8B linear-shape sweep, qkv 4096->6144, o_proj 4096->4096, "
                                "gate_up 4096->28672, down 14336->4096; M in {1,2,4,...,4096}; LUT-switched DynamicLinear.forward",
                    "group_size": 128, "layer_copies_rotated": args.copies, "lut": lut_source,
+                   "converted_weight_cache": (f"LRU, {args.resident_cache_mb} MiB" if args.resident_cache_mb > 0
+                                              else "one shared buffer (largest converted weight)"),
                    "lut_segments": prof.seg_perf_list},
         "roofline": roofline, "cpu_baseline": cpu,
         "wall_s_timed_region": round(wall, 3),

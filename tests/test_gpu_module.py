@@ -192,3 +192,37 @@ def test_checkpoint_round_trip_keeps_every_lane(gpu, cls_name, tmp_path):
         for (M, cid), ref in want.items():
             out = mod._forward(xs[M], M, cid)
             assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (cls_name, M, cid)
+
+
+def test_resident_cache_skips_conversions_and_keeps_results(gpu):
+    """Two layers alternating through the W8A8 and fp16 lanes: with the single shared buffer every call converts,
+    with an LRU cache that holds all four copies only the first call of each (layer, format) does; same bits."""
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos_amd.temp_cache import ResidentCache, TempCache
+    layers = [DynamicLinear.from_module(make_linear(256, 512, False, s)[0].cuda(), 'cuda') for s in (31, 32)]
+    x = torch.from_numpy(O.synth_acts(70, 512, seed=5)).cuda()[None]
+    lanes = (COMP_TYPE_NAME['w8a8'], COMP_TYPE_NAME['fp16'])
+
+    def run(cache, rounds=3):
+        outs = []
+        for dl in layers:
+            dl.temp_cache = cache
+        for _ in range(rounds):
+            for dl in layers:
+                for cid in lanes:
+                    outs.append(dl._forward(x, 70, cid).clone())
+        return outs
+
+    single = TempCache()
+    want = run(single)
+    assert single.hits == 0 and single.misses == 12
+    lru = ResidentCache(4 * 256 * 512 * 2)
+    got = run(lru)
+    assert lru.misses == 4 and lru.hits == 8 and lru.capacity <= lru.capacity_limit
+    small = ResidentCache(256 * 512 * 3)                     # room for one int8 and one fp16 copy: thrashes, still right
+    got_small = run(small)
+    assert small.capacity <= small.capacity_limit and small.misses > 4
+    for a, b, c in zip(want, got, got_small):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and torch.equal(a.view(torch.int16), c.view(torch.int16))
+    for dl in layers:
+        dl.temp_cache = None

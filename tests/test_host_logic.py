@@ -160,3 +160,34 @@ def test_committed_mi355x_tables_load_and_have_three_regimes():
             assert edges == sorted(edges) and all(isinstance(e, int) for e in edges)
             assert all(isinstance(s[1], str) and isinstance(s[2], float) for s in segs)
             assert segs[0][1] == "w4a16_gemv" and segs[-1][1] == "w8a8"
+
+
+def test_resident_cache_lru_and_bound():
+    from kairos_amd.temp_cache import ResidentCache, TempCache, default_cache, set_default_cache
+    c = ResidentCache(1024)
+    a, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')                     # 256 B
+    assert not hit and a.shape == (4, 64)
+    b, hit = c.get(2, 'f16', (4, 64), torch.float16, 'cpu')                  # 512 B
+    assert not hit
+    a2, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert hit and a2.data_ptr() == a.data_ptr()                             # both stay: 768 B <= 1024
+    _, hit = c.get(3, 'i8', (8, 64), torch.int8, 'cpu')                      # 512 B: evicts the least recently used (2)
+    assert not hit and c.capacity <= 1024
+    assert c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]
+    assert not c.get(2, 'f16', (4, 64), torch.float16, 'cpu')[1]             # was evicted; evicts 3 now
+    big, hit = c.get(9, 'f16', (16, 64), torch.float16, 'cpu')               # 2048 B > capacity: served, never kept
+    assert not hit and big.shape == (16, 64)
+    assert not c.get(9, 'f16', (16, 64), torch.float16, 'cpu')[1]
+    assert c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]                     # the resident entries are untouched
+    ptr = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[0].data_ptr()
+    c.invalidate()
+    again, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert not hit and again.data_ptr() == ptr                               # stale, same buffer, valid afterwards
+    assert c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]
+    assert c.peak_bytes <= 1024 + 2048 and c.hits >= 4 and c.misses >= 6
+    old = default_cache()
+    try:
+        assert set_default_cache(c) is default_cache()
+    finally:
+        set_default_cache(old)
+    assert isinstance(default_cache(), TempCache)
