@@ -3,6 +3,7 @@
     python -m kairos_amd.bench_extra gemv70b   # decode-regime W4A16 on Llama-3-70B shapes, M = 1..32
     python -m kairos_amd.bench_extra convert   # int4 -> int8 / fp16 / tiled conversion on Qwen2.5-7B shapes
     python -m kairos_amd.bench_extra decoder   # random-init Llama-3-8B decoder: TTFT / TPOT / lane switches
+    python -m kairos_amd.bench_extra blasref   # the library's int8 / fp16 GEMMs of this image (hipBLASLt via torch) beside this build's
     python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
@@ -120,6 +121,43 @@ def convert(args):
     assert cache.peak_bytes <= largest and cache.capacity <= largest, (cache.peak_bytes, cache.capacity, largest)
     return {"bench": "convert", "rows": rows, "temp_cache_peak_bytes": cache.peak_bytes,
             "largest_converted_weight_bytes": largest, "temp_cache_bounded": True}
+
+
+def blasref(args):
+    """Comparison only: the vendor library's GEMMs as shipped in this image (hipBLASLt through torch._int_mm and
+    torch.matmul) against this build's W8A8 and fp16 GEMMs on the large-M shapes of the headline benchmark, same
+    process, operands rotated.  The library's int8 GEMM writes int32 and applies no scales; this build's writes fp16
+    after the per-channel x per-token scaling.  Nothing in the product path calls the library."""
+    dev = torch.device("cuda:0")
+    rows = []
+    for M, N, K in [(4096, 4096, 4096), (4096, 6144, 4096), (4096, 28672, 4096), (4096, 4096, 14336),
+                    (1024, 28672, 4096), (1024, 4096, 4096), (512, 4096, 4096)]:
+        a8 = [torch.randint(-20, 20, (M, K), device=dev, dtype=torch.int8) for _ in range(2)]
+        w8 = [torch.randint(-20, 20, (N, K), device=dev, dtype=torch.int8) for _ in range(2)]
+        x = [a.to(torch.float16) for a in a8]
+        w16 = [w.to(torch.float16) for w in w8]
+        ws = torch.rand(N, device=dev, dtype=torch.float16)
+        asc = torch.rand(M, device=dev, dtype=torch.float16)
+        out = torch.empty((M, N), device=dev, dtype=torch.float16)
+        qw = torch.randint(-32768, 32767, (N // 4, K), device=dev, dtype=torch.int16)
+        gp = (K // G + 7) // 8 * 8
+        one = torch.ones((gp, N), device=dev, dtype=torch.float16)
+        w8t, w16t = torch.empty_like(w8[0]), torch.empty_like(w16[0])
+        ops.dequant_interleaved_int4_to_int8(w8t, qw, one, -8.0 * one, G, tiled=True)
+        ops.dequant_interleaved_int4_to_fp16(w16t, qw, one, -8.0 * one, G, tiled=True)
+        us = {"lib_i8": _time(lambda i: torch._int_mm(a8[i & 1], w8[i & 1].t()), 20),
+              "own_i8_rowmajor": _time(lambda i: ops.w8a8_gemm_forward(a8[i & 1], w8[i & 1], ws, asc, out), 20),
+              "own_i8_tiled": _time(lambda i: ops.w8a8_gemm_forward(a8[i & 1], w8t, ws, asc, out, tiled=True), 20),
+              "lib_f16": _time(lambda i: torch.matmul(x[i & 1], w16[i & 1].t()), 20),
+              "own_f16_tiled": _time(lambda i: ops.f16_gemm_forward(x[i & 1], w16t, N, tiled=True), 20)}
+        row = {"M": M, "N": N, "K": K}
+        for k, v in us.items():
+            peak = 5.0e15 if "i8" in k else 2.5e15
+            row[k + "_us"] = round(v, 1)
+            row[k + "_frac"] = round(2.0 * M * N * K / v / 1e-6 / peak, 3)
+        rows.append(row)
+        print(row, file=sys.stderr, flush=True)
+    return {"bench": "blasref", "rows": rows, "library": "hipBLASLt/rocBLAS of the image via torch %s" % torch.__version__}
 
 
 def weightprep(args):
@@ -280,6 +318,7 @@ def main(argv=None):
     sub.add_parser("gemv70b")
     sub.add_parser("convert")
     sub.add_parser("weightprep")
+    sub.add_parser("blasref")
     d = sub.add_parser("decoder")
     d.add_argument("--lut", default=None)
     d.add_argument("--layers", type=int, default=32)
@@ -294,7 +333,7 @@ def main(argv=None):
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
     ops.ensure_workspace()
-    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 
