@@ -650,12 +650,15 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         rsz[S] = szp[(long)(g >> 1) * N];
     };
 
-    // Wait until the loads of the k-tile about to be used have landed (the PF-1 younger k-tiles may stay
-    // in flight: OPS instructions each, issued in whole groups), then meet the other waves: after the
-    // barrier that k-tile's activations are complete and the previous one's stage is free.
+    // Software pipeline inside the wave: iteration j runs the MFMAs of k-tile j on weights decoded during
+    // iteration j-1 and meanwhile decodes k-tile j+1, so the decode's VALU work is spread between the MFMAs
+    // instead of standing in front of them.  At the top of iteration j every load of k-tile j+1 must have
+    // landed -- its weights and scales for the decode, its activations for the fragment reads issued during
+    // k-step 3 -- while the PF-2 younger k-tiles may stay in flight (OPS instructions each, issued in whole
+    // groups); the barrier also frees the LDS stage of k-tile j-1 for the loads of k-tile j+PF.
 #define KMI_WP_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
-    auto tile_barrier = [&]() {
-        constexpr int KEEP = (PF - 1) * OPS;
+    auto tile_barrier = [&](auto keep_tiles) {
+        constexpr int KEEP = decltype(keep_tiles)::value * OPS;
         static_assert(KEEP == 6 || KEEP == 8 || KEEP == 9 || KEEP == 12 || KEEP == 18, "no immediate for this depth");
         if constexpr (KEEP == 6) KMI_WP_BARRIER(6);
         else if constexpr (KEEP == 8) KMI_WP_BARRIER(8);
@@ -666,48 +669,84 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
 
     const int fr = lane & 31;
     const NibConsts nc = nib_consts();
-    auto body = [&](auto set, int j) {
-        constexpr int S = decltype(set)::value;
-        tile_barrier();
-        // all activation fragments of the k-tile first: the decode below covers the LDS round trip
+    u4_t pl[2][4];                                   // decoded weights: [parity of the k-tile][MFMA of the k-tile]
+    u4_t fa[2][FM];                                  // activation fragments: [parity of the k-step]
+    // pl[.][jj] covers k-step {0, 2, 1, 3}[jj]
+    auto read_frags = [&](int j, int jj, int set) {
+        const int ks = (jj == 1) ? 2 : (jj == 2) ? 1 : jj;
         const char* st = ring + (j % NSA) * A_STAGE;
-        u4_t fa[4][FM];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+        for (int i = 0; i < FM; ++i) fa[set][i] = *reinterpret_cast<const u4_t*>(st + lds_off(i * 32 + fr, 2 * ks + hl));
+    };
+    // planes 2*half, 2*half+1 of k-tile set S -> pl[par][2*half .. 2*half+1]; lower lanes keep the even plane of
+    // both chunks, upper lanes the odd one
+    auto decode_half = [&](auto set, auto half, int par, h2_t s2, h2_t z2) {
+        constexpr int S = decltype(set)::value, H = decltype(half)::value;
+        const u4_t raw = rb[S];
+        const u4_t e = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H>(raw, s2, z2, nc));
+        const u4_t o = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H + 1>(raw, s2, z2, nc));
 #pragma unroll
-            for (int i = 0; i < FM; ++i) fa[ks][i] = *reinterpret_cast<const u4_t*>(st + lds_off(i * 32 + fr, 2 * ks + hl));
-        // decode this lane's chunk: planes 0..3 = k 8a..8a+7 of its 32-wide half of the k-tile
+        for (int w = 0; w < 4; ++w) {
+            const auto x = __builtin_amdgcn_permlane32_swap(e[w], o[w], false, false);
+            pl[par][2 * H][w] = x[0];
+            pl[par][2 * H + 1][w] = x[1];
+        }
+    };
+    auto scales_of = [&](auto set, h2_t& s2, h2_t& z2) {
+        constexpr int S = decltype(set)::value;
         const uint32_t own = (uint32_t)__builtin_bit_cast(unsigned short, rsz[S]);
         const auto sw = __builtin_amdgcn_permlane32_swap(own, own, false, false);
         const uint32_t sbits = sw[0], zbits = sw[1];          // scale / scaled zero in every lane
-        const h2_t s2 = as_h2(sbits | (sbits << 16)), z2 = as_h2(zbits | (zbits << 16));
-        const u4_t raw = rb[S];
-        u4_t pl[4];
-        pl[0] = __builtin_bit_cast(u4_t, dequant_nibble_r<0>(raw, s2, z2, nc));
-        pl[1] = __builtin_bit_cast(u4_t, dequant_nibble_r<1>(raw, s2, z2, nc));
-        pl[2] = __builtin_bit_cast(u4_t, dequant_nibble_r<2>(raw, s2, z2, nc));
-        pl[3] = __builtin_bit_cast(u4_t, dequant_nibble_r<3>(raw, s2, z2, nc));
-        // lower lanes keep planes 0, 2 of both chunks, upper lanes planes 1, 3
+        s2 = as_h2(sbits | (sbits << 16));
+        z2 = as_h2(zbits | (zbits << 16));
+    };
+    auto mfma_block = [&](int par, int jj, int set) {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t a0 = pl[0][w], a1 = pl[1][w], a2 = pl[2][w], a3 = pl[3][w];
-            const auto x01 = __builtin_amdgcn_permlane32_swap(a0, a1, false, false);
-            const auto x23 = __builtin_amdgcn_permlane32_swap(a2, a3, false, false);
-            pl[0][w] = x01[0]; pl[1][w] = x01[1];
-            pl[2][w] = x23[0]; pl[3][w] = x23[1];
+        for (int i = 0; i < FM; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, pl[par][jj]), __builtin_bit_cast(h8_t, fa[set][i]),
+                                                            acc[i], 0, 0, 0);
+    };
+    // one MFMA, then a share of the other work of the block
+    auto interleave = [&](auto valu, auto ds, auto vmem) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (decltype(valu)::value > 0) __builtin_amdgcn_sched_group_barrier(0x002, (decltype(valu)::value + FM - 1) / FM, 0);
+            if constexpr (decltype(ds)::value > 0) __builtin_amdgcn_sched_group_barrier(0x100, (decltype(ds)::value + FM - 1) / FM, 0);
+            if constexpr (decltype(vmem)::value > 0) __builtin_amdgcn_sched_group_barrier(0x010, (decltype(vmem)::value + FM - 1) / FM, 0);
         }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    // iteration j: S = j % PF (compile time); weights of k-tile j are in pl[S & 1], fa[0] holds its k-step 0
+    auto body = [&](auto set, int j) {
+        constexpr int S = decltype(set)::value, SN = (S + 1) % PF, par = S & 1;
+        using SetN = std::integral_constant<int, SN>;
+        tile_barrier(std::integral_constant<int, PF - 2>{});
+        h2_t s2, z2;
+        scales_of(SetN{}, s2, z2);
+        // k-step 0 under the first half of the next decode
+        read_frags(j, 1, 1);
+        mfma_block(par, 0, 0);
+        decode_half(SetN{}, I0{}, par ^ 1, s2, z2);
+        interleave(std::integral_constant<int, 36>{}, std::integral_constant<int, FM>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
-        issue(set, j + PF);                                  // refills the registers just consumed
+        // k-step 1 under the second half
+        read_frags(j, 2, 0);
+        mfma_block(par, 1, 1);
+        decode_half(SetN{}, I1{}, par ^ 1, s2, z2);
+        interleave(std::integral_constant<int, 44>{}, std::integral_constant<int, FM>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
-        // pl[jj] covers k-step {0, 2, 1, 3}[jj]
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const int ks = (jj == 1) ? 2 : (jj == 2) ? 1 : jj;
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, pl[jj]), __builtin_bit_cast(h8_t, fa[ks][i]),
-                                                                acc[i], 0, 0, 0);
-        }
+        // k-step 2 under the loads of k-tile j+PF (their registers and their LDS stage are free now)
+        read_frags(j, 3, 1);
+        mfma_block(par, 2, 0);
+        issue(set, j + PF);
+        interleave(I0{}, std::integral_constant<int, FM>{}, std::integral_constant<int, OPS>{});
+        __builtin_amdgcn_sched_barrier(0);
+        // k-step 3 under the first fragment reads of k-tile j+1
+        read_frags(j + 1, 0, 0);
+        mfma_block(par, 3, 1);
+        interleave(I0{}, std::integral_constant<int, FM>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -719,18 +758,27 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         if constexpr (PF > 1) prime(std::integral_constant<int, 1>{});
         if constexpr (PF > 2) prime(std::integral_constant<int, 2>{});
         if constexpr (PF > 3) prime(std::integral_constant<int, 3>{});
-        static_assert(PF >= 2 && PF <= 4, "prefetch depth 2..4");
+        static_assert(PF == 4, "the loop below is unrolled for four register sets");
+    }
+    {   // k-tile 0: decoded in the open
+        tile_barrier(std::integral_constant<int, PF - 1>{});
+        h2_t s2, z2;
+        scales_of(I0{}, s2, z2);
+        decode_half(I0{}, I0{}, 0, s2, z2);
+        decode_half(I0{}, I1{}, 0, s2, z2);
+        read_frags(0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
     int j = 0;
     for (; j + PF <= T; j += PF) {
         body(std::integral_constant<int, 0>{}, j);
-        if constexpr (PF > 1) body(std::integral_constant<int, 1>{}, j + 1);
-        if constexpr (PF > 2) body(std::integral_constant<int, 2>{}, j + 2);
-        if constexpr (PF > 3) body(std::integral_constant<int, 3>{}, j + 3);
+        body(std::integral_constant<int, 1>{}, j + 1);
+        body(std::integral_constant<int, 2>{}, j + 2);
+        body(std::integral_constant<int, 3>{}, j + 3);
     }
     if (j < T) { body(std::integral_constant<int, 0>{}, j); ++j; }
-    if constexpr (PF > 2) if (j < T) { body(std::integral_constant<int, 1>{}, j); ++j; }
-    if constexpr (PF > 3) if (j < T) { body(std::integral_constant<int, 2>{}, j); ++j; }
+    if (j < T) { body(std::integral_constant<int, 1>{}, j); ++j; }
+    if (j < T) { body(std::integral_constant<int, 2>{}, j); ++j; }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // no load outlives its stage
 #undef KMI_WP_BARRIER
 
