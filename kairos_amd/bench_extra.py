@@ -206,21 +206,28 @@ class _RMSNorm(torch.nn.Module):
         self.weight = torch.ones(dim, dtype=torch.float16, device=dev)
 
     def forward(self, x):
-        v = x.float()
-        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).to(torch.float16) * self.weight
+        return torch.nn.functional.rms_norm(x, (x.shape[-1],), self.weight, 1e-5)
 
 
-def _rope(x, pos, theta=500000.0):
-    # x [B, H, S, D]; rotate-half formulation
-    d = x.shape[-1]
-    inv = 1.0 / (theta ** (torch.arange(0, d, 2, device=x.device, dtype=torch.float32) / d))
+def _rope_table(pos, d, dev, theta=500000.0):
+    """cos / sin [S, d/2] in fp16 for the positions `pos` (a device tensor): once per step, shared by all layers."""
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d))
     ang = pos.float()[:, None] * inv[None, :]
-    cos, sin = torch.cos(ang).to(x.dtype), torch.sin(ang).to(x.dtype)
+    return torch.cos(ang).to(torch.float16), torch.sin(ang).to(torch.float16)
+
+
+def _rope(x, cs):
+    # x [B, S, heads, D]; rotate-half formulation; cs = (cos, sin) [S, D/2]
+    cos, sin = cs[0][None, :, None, :], cs[1][None, :, None, :]
+    d = x.shape[-1]
     x1, x2 = x[..., : d // 2], x[..., d // 2:]
     return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
 
 
 class _Layer(torch.nn.Module):
+    """Pre-norm decoder layer over a static KV cache [B, kv_heads, T_max, d]: prefill fills positions 0..S-1, a
+    decode step writes position `pos` (a device tensor, so the step is capturable) and attends under a mask."""
+
     def __init__(self, lin, dev, hidden=4096, heads=32, kv_heads=8):
         super().__init__()
         self.h, self.kv, self.d = heads, kv_heads, hidden // heads
@@ -228,31 +235,51 @@ class _Layer(torch.nn.Module):
         self.n1, self.n2 = _RMSNorm(hidden, dev), _RMSNorm(hidden, dev)
         self.k_cache = self.v_cache = None
 
-    def forward(self, x, pos0):
+    def alloc_cache(self, B, t_max, dev):
+        self.k_cache = torch.zeros((B, self.kv, t_max, self.d), dtype=torch.float16, device=dev)
+        self.v_cache = torch.zeros_like(self.k_cache)
+
+    def _qkv(self, x, cs):
         B, S, _ = x.shape
-        qkv = self.qkv(self.n1(x))
-        q, k, v = qkv.split([self.h * self.d, self.kv * self.d, self.kv * self.d], dim=-1)
-        q = q.view(B, S, self.h, self.d).transpose(1, 2)
-        k = k.view(B, S, self.kv, self.d).transpose(1, 2)
-        v = v.view(B, S, self.kv, self.d).transpose(1, 2)
-        pos = torch.arange(pos0, pos0 + S, device=x.device)
-        q, k = _rope(q, pos), _rope(k, pos)
-        if pos0 == 0:
-            self.k_cache, self.v_cache = k, v
-        else:
-            self.k_cache = torch.cat([self.k_cache, k], dim=2)
-            self.v_cache = torch.cat([self.v_cache, v], dim=2)
-        a = torch.nn.functional.scaled_dot_product_attention(q, self.k_cache, self.v_cache, is_causal=(pos0 == 0 and S > 1),
-                                                             enable_gqa=True)
+        qkv = self.qkv(self.n1(x)).view(B, S, self.h + 2 * self.kv, self.d)
+        qk = _rope(qkv[:, :, : self.h + self.kv], cs)                      # queries and keys rotated in one pass
+        return (qk[:, :, : self.h].transpose(1, 2), qk[:, :, self.h:].transpose(1, 2),
+                qkv[:, :, self.h + self.kv:].transpose(1, 2))
+
+    def _mlp(self, x, a):
+        B, S, _ = x.shape
         x = x + self.o(a.transpose(1, 2).reshape(B, S, -1))
-        gu = self.gate_up(self.n2(x))
-        g, u = gu.chunk(2, dim=-1)
+        g, u = self.gate_up(self.n2(x)).chunk(2, dim=-1)
         return x + self.down(torch.nn.functional.silu(g) * u)
+
+    def prefill(self, x):
+        S = x.shape[1]
+        q, k, v = self._qkv(x, _rope_table(torch.arange(S, device=x.device), self.d, x.device))
+        self.k_cache[:, :, :S] = k
+        self.v_cache[:, :, :S] = v
+        a = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=S > 1, enable_gqa=True)
+        return self._mlp(x, a)
+
+    def step(self, x, pos, mask, cs):
+        """x [B, 1, hidden]; pos int64 [1] on the device; mask bool [1, 1, 1, T_max], true up to pos; cs = rope table of pos."""
+        q, k, v = self._qkv(x, cs)
+        self.k_cache.index_copy_(2, pos, k)
+        self.v_cache.index_copy_(2, pos, v)
+        # grouped-query attention of one new token, written out so that the cache is read once and never expanded
+        B, g = x.shape[0], self.h // self.kv
+        qg = q.reshape(B, self.kv, g, self.d)                               # heads of a group share one kv head
+        sc = torch.matmul(qg, self.k_cache.transpose(2, 3)) * (self.d ** -0.5)   # [B, kv, g, T_max]
+        sc = sc.masked_fill(~mask, float("-inf"))
+        a = torch.matmul(torch.softmax(sc, dim=-1, dtype=torch.float32).to(torch.float16), self.v_cache)
+        return self._mlp(x, a.view(B, self.h, 1, self.d))
 
 
 def decoder(args):
     """BASELINE config 5: 32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336, vocab 128256; every linear a
-    LUT-switched DynamicLinear (fused qkv and gate_up); protocol of utils/perf_eval.py:235-275."""
+    LUT-switched DynamicLinear (fused qkv and gate_up); protocol of utils/perf_eval.py:235-275.  The decode step
+    (all layers, final norm, vocabulary projection, greedy pick, next embedding) has fixed shapes, so it is
+    captured once per batch size into a HIP graph and replayed per token; the first tokens of every batch are
+    also generated eagerly and must agree with the replays token for token."""
     dev = torch.device("cuda:0")
     shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
     prof = Profiler(shapes)
@@ -265,50 +292,104 @@ def decoder(args):
     emb = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
     head = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
     fnorm = _RMSNorm(4096, dev)
+    t_max = args.prompt + args.new_tokens + 8
+    ar = torch.arange(t_max, device=dev)
+    names = {v: k for k, v in COMP_TYPE_NAME.items()}
 
     @torch.no_grad()
-    def generate(ids, new_tokens):
-        x = emb[ids]
-        pos = 0
-        for _ in range(new_tokens):
-            h = x
-            for L in layers:
-                h = L(h, pos)
-            pos += x.shape[1]
-            logits = fnorm(h[:, -1:, :]) @ head.T
-            nxt = logits.argmax(-1)
-            x = emb[nxt]
-        torch.cuda.synchronize()
+    def prefill(ids):
+        h = emb[ids]
+        for L in layers:
+            h = L.prefill(h)
+        return (fnorm(h[:, -1:, :]) @ head.T).argmax(-1)                  # [B, 1]
 
     results = []
     for B in args.batches:
+        for L in layers:
+            L.alloc_cache(B, t_max, dev)
         ids = torch.randint(0, vocab, (B, args.prompt), device=dev)
+        x_in = torch.zeros((B, 1, 4096), dtype=torch.float16, device=dev)   # static buffers of the step
+        pos = torch.zeros((1,), dtype=torch.int64, device=dev)
+        tok = torch.zeros((B, 1), dtype=torch.int64, device=dev)
+
+        @torch.no_grad()
+        def step():
+            mask = (ar <= pos).view(1, 1, 1, t_max)
+            cs = _rope_table(pos, 128, dev)
+            h = x_in
+            for L in layers:
+                h = L.step(h, pos, mask, cs)
+            nxt = (fnorm(h) @ head.T).argmax(-1)
+            tok.copy_(nxt)
+            x_in.copy_(emb[nxt])
+            pos.add_(1)
+
+        def start(first):
+            x_in.copy_(emb[first])
+            pos.fill_(args.prompt)
+
+        first = prefill(ids)                                                # warm-up of the prefill lanes
+        torch.cuda.synchronize()
+        start(first)
+        eager = []
+        for _ in range(args.check_tokens):                                  # also warms the decode lanes up
+            step()
+            eager.append(tok.clone())
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = None
+        if not args.eager_decode:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            start(first)
+            agree = True
+            for t in range(args.check_tokens):
+                graph.replay()
+                agree = agree and bool(torch.equal(tok, eager[t]))
+            torch.cuda.synchronize()
+            if not agree:
+                raise RuntimeError(f"decoder: graph replay and eager decoding disagree at batch {B}")
+        run_step = graph.replay if graph is not None else step
+
         for L in layers:
             for lin in (L.qkv, L.o, L.gate_up, L.down):
                 lin.switch_count = 0
-        generate(ids, 2)                                                   # warm-up
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.ttft_times):
-            generate(ids, 1)
+            first = prefill(ids)
+            torch.cuda.synchronize()
         ttft = (time.perf_counter() - t0) / args.ttft_times
-        for L in layers:
-            for lin in (L.qkv, L.o, L.gate_up, L.down):
-                lin.switch_count = 0
         t0 = time.perf_counter()
-        generate(ids, args.new_tokens)
+        first = prefill(ids)
+        start(first)
+        for _ in range(args.new_tokens - 1):
+            run_step()
+        torch.cuda.synchronize()
         total = time.perf_counter() - t0
         tpot = (total - ttft) / max(1, args.new_tokens - 1)
         sw = [sum(getattr(L, n).switch_count for L in layers) / nl for n in ("qkv", "o", "gate_up", "down")]
         results.append({"batch": B, "ttft_ms": round(ttft * 1e3, 2), "tpot_ms": round(tpot * 1e3, 3),
                         "tokens_per_s": round(B * args.new_tokens / total, 1),
-                        "switches_per_layer": {"qkv": sw[0], "o_proj": sw[1], "gate_up": sw[2], "down": sw[3]},
-                        "prefill_lane": {n: {v: k for k, v in COMP_TYPE_NAME.items()}[prof.get_comp_type(s, B * args.prompt)]
+                        "decode": "eager" if graph is None else f"HIP-graph replay, first {args.check_tokens} tokens equal to eager",
+                        "switches_per_layer_eager_calls": {"qkv": sw[0], "o_proj": sw[1], "gate_up": sw[2], "down": sw[3]},
+                        "prefill_lane": {n: names[prof.get_comp_type(s, B * args.prompt)]
                                          for n, s in zip(("qkv", "o_proj", "gate_up", "down"), shapes)},
-                        "decode_lane": {n: {v: k for k, v in COMP_TYPE_NAME.items()}[prof.get_comp_type(s, B)]
+                        "decode_lane": {n: names[prof.get_comp_type(s, B)]
                                         for n, s in zip(("qkv", "o_proj", "gate_up", "down"), shapes)}})
         print(results[-1], file=sys.stderr, flush=True)
+        del graph
+        for L in layers:
+            L.k_cache = L.v_cache = None
+        torch.cuda.empty_cache()
     return {"bench": "decoder", "layers": nl, "prompt": args.prompt, "new_tokens": args.new_tokens,
-            "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention and norms in PyTorch, greedy decoding",
+            "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention and norms in PyTorch over a static KV "
+                    "cache, greedy decoding",
             "peak_hbm_gb": round(torch.cuda.max_memory_allocated() / 1e9, 2), "rows": results}
 
 
@@ -326,6 +407,8 @@ def main(argv=None):
     d.add_argument("--new-tokens", type=int, default=512)
     d.add_argument("--ttft-times", type=int, default=3)
     d.add_argument("--batches", type=int, nargs="+", default=[2, 4, 8, 16, 32])
+    d.add_argument("--eager-decode", action="store_true", help="step token by token from Python instead of replaying a HIP graph")
+    d.add_argument("--check-tokens", type=int, default=8, help="tokens generated both eagerly and by replay, compared")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("bench_extra: needs a GPU (the HIP library is the only compute path)")
