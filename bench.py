@@ -73,7 +73,7 @@ class Tracer:
         if name == "gemm_w4a16" and self.ops.gemm_w4a16_wp_rows(M, N, K):
             label = f"{name}[wp{self.ops.gemm_w4a16_wp_rows(M, N, K)}]"
         elif name.startswith("gemm_"):
-            label = f"{name}[{self.ops.gemm_tile_for(M, N)}]"
+            label = f"{name}[{self.ops.gemm_tile_for(M, N, K)}]"
         ev = self.torch.cuda.Event(enable_timing=True)
         ev.record()
         self._cur = (label, name, M, N, K, ev)

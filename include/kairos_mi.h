@@ -161,10 +161,9 @@ int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, 
 
 /* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128 or 256. */
 void kmi_gemm_force_tile(int tile);
-/* The workgroup tile (64, 128 or 256 rows) the automatic choice uses for an M x N output.  With the 256 tile
- * the library may run the columns of a thin last round of tiles with the 128 tile in a second launch on the
- * same stream (same results). */
-int kmi_gemm_pick_tile(int M, int N);
+/* The workgroup tile (64, 128 or 256 rows) the automatic choice of the W8A8 lane uses for an M x N x K product.  With the 256 tile the library may run the columns of a
+ * thin last round of tiles with the 128 tile in a second launch on the same stream (same results). */
+int kmi_gemm_pick_tile(int M, int N, int K);
 
 /* Rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses for an M x N x K product (weights decoded
  * in registers by the wave that owns their columns), or 0 when the LDS-staged variant runs.  Forcing: tile

@@ -36,7 +36,7 @@ SIGNATURES = {
     "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kmi_gemm_force_tile": [_I],
-    "kmi_gemm_pick_tile": [_I, _I],
+    "kmi_gemm_pick_tile": [_I, _I, _I],
     "kmi_gemm_w4a16_wp_rows": [_I, _I, _I],
     "kmi_gemm_set_workspace": [_P, ctypes.c_size_t],
     "kmi_gemm_force_splits": [_I],

@@ -1152,14 +1152,19 @@ static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
     return KMI_OK;
 }
 
-// Tile choice: the largest tile that still yields about one workgroup per CU.
-static int pick_tile(int M, int N) {
+// Tile choice: the largest tile that still yields about one workgroup per CU.  row_bytes = K for the int8-operand
+// kinds.  Measured on MI355X (W8A8, tiled weights): with short rows 128 workgroups of
+// the 128 tile lose to 256 of the 64-row tile (512 x 4096 x 4096: 21.1 against 15.9 us) and win from ~144 on; with
+// long rows the 128 tile wins as soon as it yields 64 workgroups (384 x 4096 x 14336: 36.0 against 43.7 us).
+// The other kinds keep the plain rule (at least 128 workgroups of the 128 tile): row_bytes = 0.
+static int pick_tile(int M, int N, long row_bytes) {
     auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (M > 128 && wgs(256, 256) >= 180) return 256;
-    if (M > 64 && wgs(128, 128) >= 128) return 128;
+    const long need128 = row_bytes <= 0 ? 128 : row_bytes >= 8192 ? 64 : 144;
+    if (M > 64 && wgs(128, 128) >= need128) return 128;
     return 64;
 }
-extern "C" int kmi_gemm_pick_tile(int M, int N) { return pick_tile(M, N); }
+extern "C" int kmi_gemm_pick_tile(int M, int N, int K) { return pick_tile(M, N, K); }
 
 // Variant of the wave-private-weights W4A16 kernel for an M x N x K product: rows per tile (0 = run the
 // register-staged kernel instead) and wave quartets per workgroup.  Measured on MI355X (Llama-3-8B shapes):
@@ -1183,7 +1188,7 @@ extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N, int K) { return pick_wp(M, N
 
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
-    const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N);
+    const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N, (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC) ? (long)a.K : 0);
     if (tile == 256 && force_tile == 0) {
         // Round quantisation: TM x TN tiles run in rounds of 256 (one workgroup per CU).  When the last
         // round would be at most ~60 % full, the columns it would cover are run with the 128x128 tile

@@ -226,9 +226,9 @@ def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
     return out
 
 
-def gemm_tile_for(M, N):
-    """Workgroup tile (64/128/256) the automatic choice uses for an M x N output."""
-    return _lib.load().kmi_gemm_pick_tile(int(M), int(N))
+def gemm_tile_for(M, N, K=4096):
+    """Workgroup tile (64/128/256) the automatic choice uses for an M x N output over int8 rows of K bytes."""
+    return _lib.load().kmi_gemm_pick_tile(int(M), int(N), int(K))
 
 
 def gemm_w4a16_wp_rows(M, N, K=4096):
