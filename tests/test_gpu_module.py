@@ -226,3 +226,43 @@ def test_resident_cache_skips_conversions_and_keeps_results(gpu):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and torch.equal(a.view(torch.int16), c.view(torch.int16))
     for dl in layers:
         dl.temp_cache = None
+
+
+def test_quantized_llama_matches_dequantised_model(gpu):
+    """Model surgery end to end (kairos/quant_model.py:29-56) on a tiny random Llama from transformers: the logits of
+    the quantised model, with the table sending a short prompt to the small-M lane and a longer one to the W4A16
+    GEMM, match an fp16 model whose linear weights are the oracle's dequantised weights; the W8A8 lane (activations
+    quantised as well) stays within the looser bound its int8 activations imply."""
+    transformers = pytest.importorskip("transformers")
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.perf_profiler import Profiler
+    from kairos.quant_model import get_name_linears, quantize_model
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=128, max_position_embeddings=256)
+    model = transformers.LlamaForCausalLM(cfg).half().cuda().eval()
+    ref = transformers.LlamaForCausalLM(cfg).half().cuda().eval()
+    ref.load_state_dict(model.state_dict())
+    for layer in ref.model.layers:                       # the reference model computes with what the int4 tensors hold
+        for m in get_name_linears(layer).values():
+            p = O.prepare_weights(m.weight.detach().cpu().numpy())
+            m.weight.data.copy_(torch.from_numpy(O.dequant_to_f16(p["qweight"], p["scales"], p["scaled_zeros"])))
+    shapes = sorted({tuple(m.weight.shape) for layer in model.model.layers for m in get_name_linears(layer).values()})
+    prof = Profiler(shapes)
+    for s in shapes:
+        for r, name in [(8, 'w4a16_gemv'), (64, 'w4a16_gemm'), (4096, 'w8a8')]:
+            prof.record_best_comp(s, r, name)
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        quantize_model(model)
+        with torch.no_grad():
+            for T, tol in ((5, 1e-2), (40, 1e-2), (100, 6e-2)):
+                ids = torch.randint(0, 128, (1, T), device="cuda", generator=torch.Generator(device="cuda").manual_seed(T))
+                got = model(ids).logits.float()
+                want = ref(ids).logits.float()
+                assert torch.isfinite(got).all()
+                err = ((got - want).abs().max() / want.abs().max()).item()
+                assert err < tol, (T, err)
+    finally:
+        DynamicLinear.prof = old

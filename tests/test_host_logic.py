@@ -191,3 +191,48 @@ def test_resident_cache_lru_and_bound():
     finally:
         set_default_cache(old)
     assert isinstance(default_cache(), TempCache)
+
+
+def _tiny_llama(seed=0):
+    transformers = pytest.importorskip("transformers")
+    torch.manual_seed(seed)
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=128, max_position_embeddings=64)
+    return transformers.LlamaForCausalLM(cfg).half()
+
+
+def test_quantize_model_surgery_and_checkpoint_flow(tmp_path):
+    """kairos/quant_model.py:29-56 on a tiny random Llama: every decoder linear becomes a DynamicLinear whose tensors
+    equal the oracle's preparation of that weight; the dumped state_dict loads into an init_only rebuild
+    (kairos/main.py:85-91, utils/load_model.py:15-29)."""
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.quant_model import get_name_linears, quantize_model
+    from kairos.quant_config import LinearQuantConfig
+    from kairos_amd.dynamic_linear import RESIDENT_KEYS
+    model = _tiny_llama()
+    weights = {(i, n): m.weight.detach().clone() for i, layer in enumerate(model.model.layers)
+               for n, m in get_name_linears(layer).items()}
+    assert len(weights) == 14
+    cfg = quantize_model(model)
+    assert cfg == [{n: 'DynamicLinear' for n in ('self_attn.q_proj', 'self_attn.k_proj', 'self_attn.v_proj', 'self_attn.o_proj',
+                                                 'mlp.gate_proj', 'mlp.up_proj', 'mlp.down_proj')}] * 2
+    assert all(not get_name_linears(layer) for layer in model.model.layers)          # none left inside the layers
+    assert isinstance(model.lm_head, torch.nn.Linear)                                # outside the layers: untouched
+    for (i, n), w in weights.items():
+        q = model.model.layers[i].get_submodule(n)
+        assert type(q) is DynamicLinear and q.shape == tuple(w.shape)
+        ref = O.prepare_weights(w.numpy())
+        for k in RESIDENT_KEYS:
+            assert np.array_equal(getattr(q, k).numpy().view(np.uint16), ref[k].view(np.uint16)), (i, n, k)
+    path = tmp_path / "q_model.pt"
+    torch.save(model.state_dict(), path)
+    fresh = _tiny_llama(seed=1)
+    assert quantize_model(fresh, init_only=True, _quant_config=cfg) == cfg
+    fresh.load_state_dict(torch.load(path, weights_only=True))
+    for (i, n) in weights:
+        a, b = model.model.layers[i].get_submodule(n), fresh.model.layers[i].get_submodule(n)
+        assert all(torch.equal(getattr(a, k), getattr(b, k)) for k in RESIDENT_KEYS)
+    with pytest.raises(NotImplementedError):
+        LinearQuantConfig('W4A16Linear_Marlin')
+    with pytest.raises(ValueError):
+        LinearQuantConfig('nonsense')
