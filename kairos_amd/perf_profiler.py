@@ -7,6 +7,7 @@ run-length compresses the winners into segments.  `save`/`load` use the referenc
 `<dir>/seg_perf_list.pt`, JSON text, one list per shape of `[m_right_edge, lane_name, gain_pct]`.
 """
 import json
+import sys
 import os
 
 import torch
@@ -158,6 +159,7 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
                 orig_t = t
         gain = (orig_t - best_t) * 100 / orig_t if orig_t < float('inf') else 0.0
         perf_list.append((m, best_comp, gain))
+        print(f'  N={N} K={K} m={m}: {best_comp} {best_t * 1e3:.1f} us', file=sys.stderr, flush=True)   # progress: a shape takes minutes
     seg = compress_segments(perf_list)
     print('-' * 7 + f'N:{N:5d}  K:{K:5d}' + '-' * 7)
     for t in seg:
@@ -183,7 +185,8 @@ def main(argv=None):
     ap.add_argument("--preheat", type=int, default=20)
     ap.add_argument("--max-m", type=int, default=30720)
     args = ap.parse_args(argv)
-    grid = sorted(set([m for m in DEFAULT_INPUT_LEN if m <= args.max_m] + [1 << i for i in range(13)]))
+    # the reference's grid plus the powers of two and the half-way points of the region where the lanes cross
+    grid = sorted(set([m for m in DEFAULT_INPUT_LEN if m <= args.max_m] + [1 << i for i in range(13)] + [96, 192, 384, 768, 1536]))
     prof = Profiler(PRESETS[args.preset])
     details = []
     prof.profiling(input_len=grid, n=args.n, preheat_time=args.preheat, details=details)
