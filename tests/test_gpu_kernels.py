@@ -411,7 +411,11 @@ def test_gemm_tail_round_split(ops):
 @pytest.mark.parametrize("M,N,K,sel,splits", [
     (5, 128, 128, 1032, 0), (32, 256, 512, 1032, 0), (64, 256, 512, 1064, 0), (33, 384, 1024, 1064, 0),
     (64, 128, 4096, 1064, 2), (100, 256, 512, 1064, 0), (128, 256, 1024, 1128, 0), (48, 132, 256, 1064, 0),
-    (17, 256, 2048, 1032, 3), (300, 384, 512, 1128, 0), (1, 128, 14336, 1032, 0)])
+    (17, 256, 2048, 1032, 3), (300, 384, 512, 1128, 0), (1, 128, 14336, 1032, 0),
+    # every remainder of the four-deep software pipeline (k-tiles per quartet = 1..7), both quartet counts
+    (64, 256, 384, 1064, 0), (64, 256, 640, 1064, 0), (96, 256, 768, 1128, 0), (64, 256, 896, 1064, 0),
+    (64, 256, 128, 2064, 0), (128, 128, 384, 2128, 0), (32, 256, 640, 2032, 0), (200, 384, 896, 2128, 0),
+    (130, 260, 256, 2128, 0), (64, 128, 1792, 2064, 2)])
 def test_gemm_w4a16_wave_private(ops, M, N, K, sel, splits):
     """The small-M W4A16 variant (weights decoded in registers by the wave that owns their columns, quartets
     splitting K inside the workgroup, optional split over workgroups) against the oracle, with and without
