@@ -236,3 +236,12 @@ def test_quantize_model_surgery_and_checkpoint_flow(tmp_path):
         LinearQuantConfig('W4A16Linear_Marlin')
     with pytest.raises(ValueError):
         LinearQuantConfig('nonsense')
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU's share; asking for more must end with a message, not a wrong number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and r.stdout.strip() == "" and "--gpus 1" in r.stderr
