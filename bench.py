@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LUT-switched mixed-precision linear path on one MI355X.
 
-Workload (BASELINE.json configs[1]): the four linear shapes of one Llama-3-8B decoder layer
+Workload (the headline configuration): the four linear shapes of one Llama-3-8B decoder layer
 (qkv 4096->6144, o_proj 4096->4096, gate_up 4096->28672, down 14336->4096), M in {1,2,4,...,4096}.
 One STEP = for every M of the grid, one decoder layer's four linears through DynamicLinear.forward
 (LUT lookup -> selected HIP lane, conversion and activation quantisation included).  Weights are
@@ -173,8 +173,8 @@ def main():
                     help="also run one 1 GiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path is single-GPU by construction (every linear is independent; see the sharding note "
-              "in DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this path is measured on one GPU (every linear is independent and would shard by columns "
+              "without any exchange inside the kernels); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -363,14 +363,11 @@ def main():
                                  if r else " " * 18)
                 print(f"{lname:8s} {M:5d} " + " ".join(cells), file=sys.stderr)
 
-    out = args.out or os.path.join(ROOT, "gpurun_out", "bench_sweep.json")
-    try:
-        os.makedirs(os.path.dirname(out), exist_ok=True)
-        with open(out, "w") as fh:
+    if args.out:
+        os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
+        with open(args.out, "w") as fh:
             json.dump({"sweep": sweep, "by_m_us_per_layer": by_m, "kernels": kernels,
                        "launches": tracer.per_launch()}, fh, indent=1)
-    except OSError:
-        pass
 
     # best roofline fractions in the two regimes the targets name
     def best(pred):

@@ -70,7 +70,7 @@ def _layer(N, K, copies, dev):
 
 
 def gemv70b(args):
-    """BASELINE config 3: qkv 8192->10240, gate_up 8192->57344, down 28672->8192, M = 1..32."""
+    """Decode-regime W4A16 on Llama-3-70B shapes: qkv 8192->10240, gate_up 8192->57344, down 28672->8192, M = 1..32."""
     dev = torch.device("cuda:0")
     rows = []
     for name, N, K in [("qkv", 10240, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)]:
@@ -95,7 +95,7 @@ def gemv70b(args):
 
 
 def convert(args):
-    """BASELINE config 4: Qwen2.5-7B shapes; int4 -> int8, fp16, tiled; temp-cache high-water mark."""
+    """On-demand conversion on Qwen2.5-7B shapes; int4 -> int8, fp16, tiled; temp-cache high-water mark."""
     dev = torch.device("cuda:0")
     shapes = [("qkv", 4608, 3584), ("gate_up", 37888, 3584), ("down", 3584, 18944)]
     cache = TempCache()
@@ -275,7 +275,7 @@ class _Layer(torch.nn.Module):
 
 
 def decoder(args):
-    """BASELINE config 5: 32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336, vocab 128256; every linear a
+    """End-to-end decoder: 32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336, vocab 128256; every linear a
     LUT-switched DynamicLinear (fused qkv and gate_up); protocol of utils/perf_eval.py:235-275.  The decode step
     (all layers, final norm, vocabulary projection, greedy pick, next embedding) has fixed shapes, so it is
     captured once per batch size into a HIP graph and replayed per token; the first tokens of every batch are

@@ -451,7 +451,7 @@ def test_gemm_w4a16_variant_choice(ops):
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(48, 28672, 4096), (200, 4096, 14336)])
 def test_gemm_w4a16_variants_agree_at_full_size(ops, M, N, K):
-    """At BASELINE sizes the oracle is too slow; the two W4A16 GEMM variants (wave-private, register-staged) and
+    """At the benchmark's full sizes the oracle is too slow; the two W4A16 GEMM variants (wave-private, register-staged) and
     the small-M kernel are independent implementations of the same product and must agree within the fp16
     tolerance on random packed weights."""
     g = torch.Generator(device="cuda").manual_seed(M + N)
