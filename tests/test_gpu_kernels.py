@@ -592,3 +592,74 @@ def test_trans_layout_w4a8_rejects_bad_shapes(ops):
         ops.trans_layout_c16_to_c8_awq(t, 16, 128)          # N % 32
     with pytest.raises(ValueError):
         ops.trans_layout_c16_to_c8_awq(t, 64, 64)           # size mismatch
+
+
+# ------------------------------------------------------------------ random shapes: every variant of a lane agrees
+def test_random_shapes_every_variant_agrees(ops):
+    """Sixty random (M, N, K) with ragged N, odd M and optional bias.  W8A8: every tile, row-major and tiled weights,
+    separate and fused preparation give the same bits, and the int32 accumulators equal an exact matmul.  W4A16: every
+    kernel variant (three staged tiles, six wave-private ones, the small-M kernel) and the fp16 GEMM on converted
+    weights stay within the fp16 tolerance of an fp32 product of the converted weights."""
+    import random
+    rnd = random.Random(7)
+
+    def same(a, b):
+        return torch.equal(a.view(torch.int16) if a.dtype == torch.float16 else a,
+                           b.view(torch.int16) if b.dtype == torch.float16 else b)
+
+    for it in range(60):
+        M = rnd.choice([1, 3, 17, 33, 64, 65, 100, 128, 129, 200, 256, 257, 300, 511, 512, 700, 1024])
+        N = 4 * rnd.randint(1, 500) if rnd.random() < 0.5 else 128 * rnd.randint(1, 24)
+        K = 128 * rnd.randint(1, 20)
+        tag = f"case {it}: M={M} N={N} K={K}"
+        g = torch.Generator(device="cuda").manual_seed(it)
+        qw = torch.randint(-32768, 32767, (N // 4, K), device="cuda", dtype=torch.int16, generator=g)
+        gp = O.padded_groups(K)
+        s = (torch.rand((gp, N), device="cuda", generator=g) * 0.01 + 0.002).to(torch.float16)
+        z = (-(s.float() * 7.5)).to(torch.float16)
+        s8 = (torch.rand((gp, N), device="cuda", generator=g) * 6 + 2).to(torch.float16)
+        z8 = (-(s8.float() * 7.5)).to(torch.float16)
+        x = torch.randn((M, K), device="cuda", generator=g).to(torch.float16)
+        bias = torch.randn((N,), device="cuda", generator=g).to(torch.float16) if rnd.random() < 0.5 else None
+        w8 = torch.empty((N, K), device="cuda", dtype=torch.int8)
+        ops.dequant_interleaved_int4_to_int8(w8, qw, s8, z8, 128)
+        a8 = torch.empty((M, K), device="cuda", dtype=torch.int8)
+        sx = torch.empty((M,), device="cuda", dtype=torch.float16)
+        ops.quant_fp16_to_int8(a8, x, sx)
+        ws = torch.rand((N,), device="cuda", generator=g).to(torch.float16)
+        outs = []
+        try:
+            for tile in (0, 64, 128, 256):
+                ops.force_gemm_tile(tile)
+                o = torch.empty((M, N), device="cuda", dtype=torch.float16)
+                ops.w8a8_gemm_forward(a8, w8, ws, sx, o, bias=bias)
+                outs.append(o)
+                if N % 128 == 0:
+                    w8t, a8b, sxb = torch.empty_like(w8), torch.empty_like(a8), torch.empty_like(sx)
+                    ops.prep_w8a8(w8t, qw, s8, z8, a8b, x, sxb, 128, tiled=True)
+                    ot = torch.empty((M, N), device="cuda", dtype=torch.float16)
+                    ops.w8a8_gemm_forward(a8b, w8t, ws, sxb, ot, bias=bias, tiled=True)
+                    outs.append(ot)
+                    assert same(a8, a8b) and same(sx, sxb) and same(ops.untile(w8t, N, K), w8), tag
+        finally:
+            ops.force_gemm_tile(0)
+        assert all(same(outs[0], o) for o in outs[1:]), tag
+        assert same(ops.w8a8_gemm_acc_i32(a8, w8, N), (a8.double() @ w8.double().T).to(torch.int32)), tag
+        w16 = torch.empty((N, K), device="cuda", dtype=torch.float16)
+        ops.dequant_interleaved_int4_to_fp16(w16, qw, s, z, 128)
+        want = x.float() @ w16.float().T
+        if bias is not None:
+            want = want + bias.float()
+        scale = want.abs().max().item() + 1e-6
+        for sel in (0, 64, 128, 256, 1032, 1064, 1128, 2032, 2064, 2128):
+            ops.force_gemm_tile(sel)
+            try:
+                o = ops.gemm_forward(x, qw, s, z, bias=bias)
+            finally:
+                ops.force_gemm_tile(0)
+            assert (o.float() - want).abs().max().item() / scale < 4e-3, (tag, sel)
+        if M <= 64 and N % 16 == 0:
+            o = ops.gemv_forward(x, qw, s, z, M, N, K, 128, bias=bias)
+            assert (o.float() - want).abs().max().item() / scale < 4e-3, (tag, "small-M kernel")
+        o = ops.f16_gemm_forward(x, w16, N, bias=bias)
+        assert (o.float() - want).abs().max().item() / scale < 4e-3, (tag, "fp16 GEMM")
