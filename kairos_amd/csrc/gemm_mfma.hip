@@ -12,6 +12,8 @@
 // keeps two k-tiles in flight in two register sets and writes them to the other of two LDS stages:
 // one barrier per k-tile.  The operand-copy kinds (F16, W8A8) use gemm_direct_kernel further down:
 // direct-to-LDS loads, four 64-byte stages.
+// W4A16 products of up to ~1000 rows run gemm_w4a16_wp_kernel instead (weights decoded in registers by the wave
+// that owns their columns, never written to LDS); the host side at the end of the file picks kernel and tile.
 #include "kmi_common.h"
 #include <type_traits>
 
