@@ -245,3 +245,28 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0 and r.stdout.strip() == "" and "--gpus 1" in r.stderr
+
+
+def test_apply_scale_keeps_the_fp_function():
+    """kairos/smooth_scale.py:33-63: folding per-channel scales into the linears (W * s) and into the operator that
+    feeds them (norm weight or up_proj rows / s) leaves the layer's function unchanged; fp32 model, so the comparison
+    is tight.  The three blocks are the ones the reference's search emits (:107-131)."""
+    from kairos.smooth_scale import apply_scale
+    model = _tiny_llama(seed=3).float()
+    ids = torch.randint(0, 128, (2, 12), generator=torch.Generator().manual_seed(0))
+    with torch.no_grad():
+        before = model(ids).logits
+    g = torch.Generator().manual_seed(1)
+    meta = []
+    for _ in model.model.layers:
+        meta.append([("input_layernorm", ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"], torch.rand(1, 256, generator=g) + 0.5),
+                     ("post_attention_layernorm", ["mlp.gate_proj", "mlp.up_proj"], torch.rand(1, 256, generator=g) + 0.5),
+                     ("mlp.up_proj", ["mlp.down_proj"], torch.rand(1, 512, generator=g) + 0.5)])
+    w0 = model.model.layers[0].self_attn.q_proj.weight.detach().clone()
+    apply_scale(model, meta)
+    assert torch.allclose(model.model.layers[0].self_attn.q_proj.weight, w0 * meta[0][0][2])
+    with torch.no_grad():
+        after = model(ids).logits
+    assert torch.allclose(before, after, rtol=1e-4, atol=1e-4)
+    with pytest.raises(ValueError):
+        apply_scale(model, [[("no_such_op", ["mlp.down_proj"], torch.ones(1, 512))]])
