@@ -210,14 +210,21 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
     return nullptr;
 }
 
-// Default split, from sweeps on MI355X.  Eight waves per workgroup over K.  Column tiles per wave: for
-// M <= 8 activation traffic is negligible, so favour occupancy (two tiles); above that reuse each
-// activation fragment for four tiles -- in both cases only while about 200 workgroups remain.
+// Default split, from sweeps on MI355X over the Llama-3-8B and -70B shapes.
+//   Column tiles per wave (nt): the most of 4, 2, 1 that still leaves about 150 workgroups -- every activation
+//   fragment is reused nt times and fewer, longer workgroups stream better (10240 x 8192 at M=16: 14.7 us with
+//   nt=4 and 160 workgroups against 20.8 us with nt=2 and 320) -- except that for M <= 4 a grid that would still be
+//   several rounds of workgroups keeps nt=2 (57344 x 8192 at M=1: 42.8 against 49.7 us).
+//   Waves per workgroup over K (nw): eight; sixteen for a single column tile at the smallest M, where the kernel is
+//   a pure latency chain (4096 x 14336 at M=1: 10.4 against 11.9 us); four from three row tiles on (M > 32).
 static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_out) {
     const int strips = (N + 15) / 16, groups = K / 128;
-    int nt = (M <= 8) ? 2 : 4;
-    while (nt > 1 && ((strips + nt - 1) / nt < 192 || gemv_lookup(mt, nt, 8) == nullptr)) nt >>= 1;
+    int nt = 4;
+    if (M <= 4 && (strips + 3) / 4 > 768) nt = 2;
+    while (nt > 1 && ((strips + nt - 1) / nt < 150 || gemv_lookup(mt, nt, 8) == nullptr)) nt >>= 1;
     int nw = 8;
+    if (nt == 1 && (M <= 4 || (M <= 8 && K <= 4096)) && groups >= 16 && gemv_lookup(mt, nt, 16) != nullptr) nw = 16;
+    if (mt >= 3 && nt >= 2 && gemv_lookup(mt, nt, 4) != nullptr) nw = 4;
     while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
     *nt_out = nt;
     *nw_out = nw;
