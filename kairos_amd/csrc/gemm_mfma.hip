@@ -1169,28 +1169,54 @@ static int pick_tile(int M, int N, long row_bytes) {
 extern "C" int kmi_gemm_pick_tile(int M, int N, int K) { return pick_tile(M, N, K); }
 
 // Variant of the wave-private-weights W4A16 kernel for an M x N x K product: rows per tile (0 = run the
-// register-staged kernel instead) and wave quartets per workgroup.  Measured on MI355X (Llama-3-8B shapes):
-// the wave-private kernel wins while its tiles fit one or two rounds over the CUs; 64-row tiles while they
-// fit one round, 128-row tiles beyond that or when K is long (the decode of a weight is then shared by twice
-// as many rows), a single quartet per workgroup once there are more tiles than CUs.
+// register-staged kernel instead) and wave quartets per workgroup.  Measured on MI355X (Llama-3-8B and -70B
+// shapes): the wave-private kernel wins while its tiles fit one or two rounds over the CUs; 64-row tiles while
+// they fit one round, 128-row tiles beyond that or when K is long and there are at least 64 of them (the decode of
+// a weight is then shared by twice as many rows: 10240 x 8192 at M=128 37 against 44 us), a single quartet per
+// workgroup once there are more tiles than CUs.  Beyond two rounds the register-staged kernel takes over only
+// where it runs its 256-row tile without more row padding than 128-row tiles would have (28672 x 4096: M=512
+// 131 against 141 us for the staged kernel, M=384 126 against 109 us).  Very few tiles: 32-row tiles up to M=64
+// (4096 x 4096 at M=64: 12.5 against 13.7 us).  Where 128-row tiles would pad M further than 64-row tiles (M = 192,
+// 320, ...) the 64-row variants are preferred (37888 x 3584 at M=192: 71 against 84 us).
 struct WpChoice { int rows, quartets; };
 static WpChoice pick_wp(int M, int N, int K) {
     if (M > 1024) return {0, 0};
     const long strips = (N + 127) / 128;
-    const long tiles64 = ((M + 63) / 64) * strips, tiles128 = ((M + 127) / 128) * strips;
+    const long tiles32 = ((M + 31) / 32) * strips, tiles64 = ((M + 63) / 64) * strips, tiles128 = ((M + 127) / 128) * strips;
+    const bool pad128 = (M + 127) / 128 * 2 > (M + 63) / 64;      // 128-row tiles pad M further than 64-row tiles
     if (M <= 32) return {32, 2};
-    if (M <= 64) return {64, 2};
-    if (K >= 8192 && M > 128 && tiles128 <= 256) return {128, 2};
+    if (M <= 64) return (tiles32 <= 80 && K <= 8192) ? WpChoice{32, 2} : WpChoice{64, 2};
+    // long K: 128-row tiles from 64 tiles on, unless they pad more, cannot be split over K and 64-row tiles fit a round
+    if (K >= 8192 && tiles128 >= 64 && tiles128 <= 256 && !(pad128 && tiles128 > 128 && tiles64 <= 256)) return {128, 2};
     if (tiles64 <= 256) return {64, 2};
     if (tiles128 <= 256) return {128, 2};
+    if (pad128 && tiles64 <= 2048) return {64, 1};
     if (tiles128 <= 512) return {128, 1};
-    return {0, 0};
+    const bool staged256 = pick_tile(M, N, 0) == 256 && (M + 255) / 256 * 2 == (M + 127) / 128;
+    return staged256 ? WpChoice{0, 0} : WpChoice{128, 1};
 }
 extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N, int K) { return pick_wp(M, N, K).rows; }
 
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
     const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N, (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC) ? (long)a.K : 0);
+    if constexpr (KIND == KIND_W4A16) {
+        // selectors 1032 / 1064 / 1128 force the wave-private-weights kernel with 32 / 64 / 128 rows per tile
+        if (tile == 1032) return launch_w4a16_wp<32>(a, st);
+        if (tile == 1064) return launch_w4a16_wp<64>(a, st);
+        if (tile == 1128) return launch_w4a16_wp<128>(a, st);
+        if (tile == 2032) return launch_w4a16_wp<32, 1>(a, st);      // 2xxx: one wave quartet per workgroup
+        if (tile == 2064) return launch_w4a16_wp<64, 1>(a, st);
+        if (tile == 2128) return launch_w4a16_wp<128, 1>(a, st);
+        if (force_tile == 0) {
+            const WpChoice c = pick_wp(a.M, a.N, a.K);
+            if (c.rows == 32) return launch_w4a16_wp<32>(a, st);
+            if (c.rows == 64 && c.quartets == 2) return launch_w4a16_wp<64>(a, st);
+            if (c.rows == 64) return launch_w4a16_wp<64, 1>(a, st);
+            if (c.rows == 128 && c.quartets == 2) return launch_w4a16_wp<128>(a, st);
+            if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, st);
+        }
+    }
     if (tile == 256 && force_tile == 0) {
         // Round quantisation: TM x TN tiles run in rounds of 256 (one workgroup per CU).  When the last
         // round would be at most ~60 % full, the columns it would cover are run with the 128x128 tile
@@ -1203,22 +1229,6 @@ static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
             const int rc = launch_gemm<KIND, 256, 256, TILED>(a, st, 0, head_cols * 256);
             if (rc != KMI_OK) return rc;
             return launch_gemm<KIND, 128, 128, TILED>(a, st, head_cols * 256, a.N - head_cols * 256);
-        }
-    }
-    if constexpr (KIND == KIND_W4A16) {
-        // selectors 1032 / 1064 / 1128 force the wave-private-weights kernel with 32 / 64 / 128 rows per tile
-        if (tile == 1032) return launch_w4a16_wp<32>(a, st);
-        if (tile == 1064) return launch_w4a16_wp<64>(a, st);
-        if (tile == 1128) return launch_w4a16_wp<128>(a, st);
-        if (tile == 2032) return launch_w4a16_wp<32, 1>(a, st);      // 2xxx: one wave quartet per workgroup
-        if (tile == 2064) return launch_w4a16_wp<64, 1>(a, st);
-        if (tile == 2128) return launch_w4a16_wp<128, 1>(a, st);
-        if (force_tile == 0) {
-            const WpChoice c = pick_wp(a.M, a.N, a.K);
-            if (c.rows == 32) return launch_w4a16_wp<32>(a, st);
-            if (c.rows == 64) return launch_w4a16_wp<64>(a, st);
-            if (c.rows == 128 && c.quartets == 2) return launch_w4a16_wp<128>(a, st);
-            if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, st);
         }
     }
     switch (tile) {

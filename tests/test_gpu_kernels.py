@@ -446,6 +446,8 @@ def test_gemm_w4a16_variant_choice(ops):
     assert ops.gemm_w4a16_wp_rows(256, 6144, 4096) == 64 and ops.gemm_w4a16_wp_rows(512, 6144, 4096) == 128
     assert ops.gemm_w4a16_wp_rows(256, 4096, 14336) == 128 and ops.gemm_w4a16_wp_rows(256, 28672, 4096) == 128
     assert ops.gemm_w4a16_wp_rows(512, 28672, 4096) == 0 and ops.gemm_w4a16_wp_rows(2048, 4096, 4096) == 0
+    assert ops.gemm_w4a16_wp_rows(64, 4096, 4096) == 32 and ops.gemm_w4a16_wp_rows(384, 28672, 4096) == 128
+    assert ops.gemm_w4a16_wp_rows(128, 10240, 8192) == 128 and ops.gemm_w4a16_wp_rows(128, 4096, 14336) == 64
 
 
 @pytest.mark.gpu
