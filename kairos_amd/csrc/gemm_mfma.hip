@@ -1155,15 +1155,30 @@ static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
 }
 
 // Tile choice: the largest tile that still yields about one workgroup per CU.  row_bytes = K for the int8-operand
-// kinds.  Measured on MI355X (W8A8, tiled weights): with short rows 128 workgroups of
-// the 128 tile lose to 256 of the 64-row tile (512 x 4096 x 4096: 21.1 against 15.9 us) and win from ~144 on; with
-// long rows the 128 tile wins as soon as it yields 64 workgroups (384 x 4096 x 14336: 36.0 against 43.7 us).
-// The other kinds keep the plain rule (at least 128 workgroups of the 128 tile): row_bytes = 0.
+// kinds (0 for the others, which keep the plain rule: 256-row tiles from 180 workgroups, 128-row tiles from 128).
+// Measured on MI355X (W8A8, tiled weights, Llama-3-8B / -70B and Qwen2.5-7B shapes):
+//   * the 256 tile pays from ~144 workgroups on (256 x 37888 x 3584: 50 against 68 us with the 128 tile), and on
+//     long rows already when a split over K brings it there, provided every split keeps ~9000 bytes of K
+//     (768 x 8192 x 28672: 96 tiles x 2 splits, 189 against 284 us; 2048 x 4096 x 14336 split in two loses);
+//   * with short rows 128 workgroups of the 128 tile lose to 256 of the 64-row tile (512 x 4096 x 4096: 21.1
+//     against 15.9 us) and win from ~144 on; with long rows the 128 tile wins from ~48 workgroups
+//     (384 x 4096 x 14336: 36.0 against 43.7 us);
+//   * where 128-row tiles pad M further than 64-row tiles and would not fill the GPU while the 64-row tiles do,
+//     the latter win (192 x 10240 x 8192: 28.8 against 31.9 us; not at 192 x 28672 x 4096: 52.5 against 43.7 us).
 static int pick_tile(int M, int N, long row_bytes) {
     auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M > 128 && wgs(256, 256) >= 180) return 256;
-    const long need128 = row_bytes <= 0 ? 128 : row_bytes >= 8192 ? 64 : 144;
-    if (M > 64 && wgs(128, 128) >= need128) return 128;
+    if (row_bytes <= 0) {
+        if (M > 128 && wgs(256, 256) >= 180) return 256;
+        if (M > 64 && wgs(128, 128) >= 128) return 128;
+        return 64;
+    }
+    long split = 256 / wgs(256, 256);
+    if (split > row_bytes / 9000) split = row_bytes / 9000;
+    if (split < 1) split = 1;
+    if (M > 128 && wgs(256, 256) * split >= 144) return 256;
+    const bool pad128 = (M + 127) / 128 * 2 > (M + 63) / 64;
+    if (pad128 && wgs(64, 128) >= 200 && wgs(128, 128) < 256) return 64;
+    if (M > 64 && wgs(128, 128) >= (row_bytes >= 8192 ? 48 : 144)) return 128;
     return 64;
 }
 extern "C" int kmi_gemm_pick_tile(int M, int N, int K) { return pick_tile(M, N, K); }
