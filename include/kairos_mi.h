@@ -85,6 +85,18 @@ int kmi_quant_act_i8(void* out_i8, void* scale_f16, const void* x_f16, int M, in
 int kmi_prep_w8a8(void* w8_out, int tiled, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
                   int N, int K, int G, void* a8_out, void* ascale_f16, const void* x_f16, int M, void* stream);
 
+/* RMSNorm in front of a switched linear, emitting the activation format the consumer's lane needs from one read
+ * of the hidden state ("activation matching", README.md:23-27; the reference vendors a fused norm + per-token
+ * quantiser, thirdparty/AWQ/kernels/csrc/w8a8/layernorm.cu:51-231 `rms_norm_general`, which kairos/ never calls:
+ * its modules run the eager norm and then quant_fp16_to_int8).  With h = x, or h = fp16(x + residual) when
+ * residual_f16 is given (then also written to h_f16_out if that is not NULL):
+ *   r = 1.0f / sqrtf(sum_k float(h[m,k])^2 / K + eps);  y[m,k] = fp16(float(gamma[k]) * float(fp16(float(h[m,k]) * r)))
+ * which is the fp16 RMSNorm of the Llama / Qwen decoder modules with every intermediate rounded as there.
+ * y_f16_out (may be NULL) receives y; a8_out / ascale_f16 (may both be NULL) receive kmi_quant_act_i8 of y, bit for
+ * bit.  At least one output is required.  Needs K%8==0, K<=32768, eps>=0, 16-byte aligned tensors. */
+int kmi_rmsnorm_quant_act(void* a8_out, void* ascale_f16, void* y_f16_out, void* h_f16_out, const void* x_f16,
+                          const void* residual_f16, const void* gamma_f16, float eps, int M, int K, void* stream);
+
 /* ---- offline weight preparation ----------------------------------------------------------------- */
 
 /* fp16 weight [N, K] (row-major) -> the resident format of one linear, in one launch:

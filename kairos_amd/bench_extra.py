@@ -20,6 +20,7 @@ import numpy as np
 import torch
 
 from . import ops
+from .act_matching import MatchedRMSNorm
 from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
 from .perf_profiler import Profiler
 from .temp_cache import TempCache
@@ -226,43 +227,59 @@ def _rope(x, cs):
 
 class _Layer(torch.nn.Module):
     """Pre-norm decoder layer over a static KV cache [B, kv_heads, T_max, d]: prefill fills positions 0..S-1, a
-    decode step writes position `pos` (a device tensor, so the step is capturable) and attends under a mask."""
+    decode step writes position `pos` (a device tensor, so the step is capturable) and attends under a mask.
+    The residual stream travels as (x, delta) with hidden = x + delta: with `matched` norms the add, the norm and
+    the activation format of the consuming linear's lane come from one kernel (kairos_amd/act_matching.py)."""
 
-    def __init__(self, lin, dev, hidden=4096, heads=32, kv_heads=8):
+    def __init__(self, lin, dev, hidden=4096, heads=32, kv_heads=8, matched=True):
         super().__init__()
         self.h, self.kv, self.d = heads, kv_heads, hidden // heads
         self.qkv, self.o, self.gate_up, self.down = lin
         self.n1, self.n2 = _RMSNorm(hidden, dev), _RMSNorm(hidden, dev)
+        if matched:
+            self.n1 = MatchedRMSNorm(self.n1.weight, 1e-5, [self.qkv])
+            self.n2 = MatchedRMSNorm(self.n2.weight, 1e-5, [self.gate_up])
+        self.matched = matched
         self.k_cache = self.v_cache = None
 
     def alloc_cache(self, B, t_max, dev):
         self.k_cache = torch.zeros((B, self.kv, t_max, self.d), dtype=torch.float16, device=dev)
         self.v_cache = torch.zeros_like(self.k_cache)
 
-    def _qkv(self, x, cs):
+    def _norm(self, norm, x, delta):
+        """-> (input of the consuming linear, hidden = x + delta)"""
+        if self.matched:
+            act, h = norm(x, delta)
+            return act, (x if h is None else h)
+        h = x if delta is None else x + delta
+        return norm(h), h
+
+    def _qkv(self, x, delta, cs):
         B, S, _ = x.shape
-        qkv = self.qkv(self.n1(x)).view(B, S, self.h + 2 * self.kv, self.d)
+        y, x = self._norm(self.n1, x, delta)
+        qkv = self.qkv(y).view(B, S, self.h + 2 * self.kv, self.d)
         qk = _rope(qkv[:, :, : self.h + self.kv], cs)                      # queries and keys rotated in one pass
-        return (qk[:, :, : self.h].transpose(1, 2), qk[:, :, self.h:].transpose(1, 2),
+        return (x, qk[:, :, : self.h].transpose(1, 2), qk[:, :, self.h:].transpose(1, 2),
                 qkv[:, :, self.h + self.kv:].transpose(1, 2))
 
     def _mlp(self, x, a):
         B, S, _ = x.shape
-        x = x + self.o(a.transpose(1, 2).reshape(B, S, -1))
-        g, u = self.gate_up(self.n2(x)).chunk(2, dim=-1)
-        return x + self.down(torch.nn.functional.silu(g) * u)
+        y, x = self._norm(self.n2, x, self.o(a.transpose(1, 2).reshape(B, S, -1)))
+        g, u = self.gate_up(y).chunk(2, dim=-1)
+        return x, self.down(torch.nn.functional.silu(g) * u)
 
-    def prefill(self, x):
+    def prefill(self, x, delta):
         S = x.shape[1]
-        q, k, v = self._qkv(x, _rope_table(torch.arange(S, device=x.device), self.d, x.device))
+        x, q, k, v = self._qkv(x, delta, _rope_table(torch.arange(S, device=x.device), self.d, x.device))
         self.k_cache[:, :, :S] = k
         self.v_cache[:, :, :S] = v
         a = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=S > 1, enable_gqa=True)
         return self._mlp(x, a)
 
-    def step(self, x, pos, mask, cs):
-        """x [B, 1, hidden]; pos int64 [1] on the device; mask bool [1, 1, 1, T_max], true up to pos; cs = rope table of pos."""
-        q, k, v = self._qkv(x, cs)
+    def step(self, x, delta, pos, mask, cs):
+        """x, delta [B, 1, hidden]; pos int64 [1] on the device; mask bool [1, 1, 1, T_max], true up to pos; cs = rope
+        table of pos."""
+        x, q, k, v = self._qkv(x, delta, cs)
         self.k_cache.index_copy_(2, pos, k)
         self.v_cache.index_copy_(2, pos, v)
         # grouped-query attention of one new token, written out so that the cache is read once and never expanded
@@ -287,7 +304,7 @@ def decoder(args):
     DynamicLinear.prof = prof
     nl = args.layers
     per_shape = [_layer(N, K, nl, dev) for N, K in shapes]
-    layers = [_Layer([per_shape[s][l] for s in range(4)], dev) for l in range(nl)]
+    layers = [_Layer([per_shape[s][l] for s in range(4)], dev, matched=not args.torch_norm) for l in range(nl)]
     vocab = 128256
     emb = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
     head = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
@@ -298,10 +315,10 @@ def decoder(args):
 
     @torch.no_grad()
     def prefill(ids):
-        h = emb[ids]
+        h, delta = emb[ids], None
         for L in layers:
-            h = L.prefill(h)
-        return (fnorm(h[:, -1:, :]) @ head.T).argmax(-1)                  # [B, 1]
+            h, delta = L.prefill(h, delta)
+        return (fnorm(h[:, -1:, :] + delta[:, -1:, :]) @ head.T).argmax(-1)    # [B, 1]
 
     results = []
     for B in args.batches:
@@ -316,10 +333,10 @@ def decoder(args):
         def step():
             mask = (ar <= pos).view(1, 1, 1, t_max)
             cs = _rope_table(pos, 128, dev)
-            h = x_in
+            h, delta = x_in, None
             for L in layers:
-                h = L.step(h, pos, mask, cs)
-            nxt = (fnorm(h) @ head.T).argmax(-1)
+                h, delta = L.step(h, delta, pos, mask, cs)
+            nxt = (fnorm(h + delta) @ head.T).argmax(-1)
             tok.copy_(nxt)
             x_in.copy_(emb[nxt])
             pos.add_(1)
@@ -388,8 +405,10 @@ def decoder(args):
             L.k_cache = L.v_cache = None
         torch.cuda.empty_cache()
     return {"bench": "decoder", "layers": nl, "prompt": args.prompt, "new_tokens": args.new_tokens,
-            "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention and norms in PyTorch over a static KV "
-                    "cache, greedy decoding",
+            "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention in PyTorch over a static KV cache, "
+                    + ("norms in PyTorch" if args.torch_norm else "residual add + RMSNorm + activation format of the next lane in "
+                       "one kernel (kmi_rmsnorm_quant_act)") + ", greedy decoding",
+            "norms": "torch" if args.torch_norm else "matched",
             "peak_hbm_gb": round(torch.cuda.max_memory_allocated() / 1e9, 2), "rows": results}
 
 
@@ -408,6 +427,7 @@ def main(argv=None):
     d.add_argument("--ttft-times", type=int, default=3)
     d.add_argument("--batches", type=int, nargs="+", default=[2, 4, 8, 16, 32])
     d.add_argument("--eager-decode", action="store_true", help="step token by token from Python instead of replaying a HIP graph")
+    d.add_argument("--torch-norm", action="store_true", help="PyTorch residual adds and RMSNorms instead of the fused matched norm")
     d.add_argument("--check-tokens", type=int, default=8, help="tokens generated both eagerly and by replay, compared")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():

@@ -107,6 +107,38 @@ __device__ __forceinline__ void cvt_i4_body(long i, void* __restrict__ out, cons
     }
 }
 
+// Eight fp16 values times the token's factor t -> eight int8: q = sat_s8(round_half_even(float(v) * t)), NaN -> 0
+// (0 * inf of an all-zero token).  The conversion instruction itself maps NaN to 0 and saturates, so no compare is
+// needed; the clamp to the int8 range is an integer median; v_perm gathers the low bytes.
+__device__ __forceinline__ int cvt_rne_i32(float p) {
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(rintf(p)));
+    return q;
+}
+__device__ __forceinline__ u2_t quantise_h8(const h8_t& v, float t) {
+    uint32_t q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        int i = cvt_rne_i32((float)v[e] * t);
+        i = i < -128 ? -128 : (i > 127 ? 127 : i);
+        q[e] = (uint32_t)i;
+    }
+    u2_t o;
+    o[0] = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[3], q[2], 0x0c0c0400u), __builtin_amdgcn_perm(q[1], q[0], 0x0c0c0400u), 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[7], q[6], 0x0c0c0400u), __builtin_amdgcn_perm(q[5], q[4], 0x0c0c0400u), 0x05040100u);
+    return o;
+}
+
+// Absolute maximum of eight fp16 values, folded into `m` (packed fp16 maxima: NaN operands are ignored, as by fmaxf).
+__device__ __forceinline__ h2_t amax_h8(h2_t m, const h8_t& v) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const h2_t a = as_h2(as_u32(h2_t{v[2 * e], v[2 * e + 1]}) & 0x7fff7fffu);
+        m = __builtin_elementwise_max(m, a);
+    }
+    return m;
+}
+
 // Quantises one token with the whole 256-thread workgroup (CPT 16-byte chunks per thread).
 template <int CPT>
 __device__ __forceinline__ void quant_act_body(int token, int8_t* __restrict__ out, half_t* __restrict__ scale,
@@ -114,16 +146,16 @@ __device__ __forceinline__ void quant_act_body(int token, int8_t* __restrict__ o
     const int nchunk = K >> 3;
     const h8_t* row = reinterpret_cast<const h8_t*>(x + (long)token * K);
     h8_t v[CPT];
-    float amax = 0.0f;
+    h2_t am2 = {(half_t)0.0f, (half_t)0.0f};
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
         const int c = threadIdx.x + i * 256;
         if (c < nchunk) {
             v[i] = row[c];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)v[i][e]));
+            am2 = amax_h8(am2, v[i]);
         }
     }
+    float amax = fmaxf((float)am2[0], (float)am2[1]);
     __shared__ float red[4];
     amax = wave_max(amax);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
@@ -135,20 +167,7 @@ __device__ __forceinline__ void quant_act_body(int token, int8_t* __restrict__ o
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
         const int c = threadIdx.x + i * 256;
-        if (c < nchunk) {
-            uint32_t b[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float p = (float)v[i][e] * t;
-                p = (p != p) ? 0.0f : p;        // 0 * inf
-                p = fminf(fmaxf(rintf(p), -128.0f), 127.0f);
-                b[e] = (uint32_t)(uint8_t)(int8_t)(int)p;
-            }
-            u2_t o;
-            o[0] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-            o[1] = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
-            orow[c] = o;
-        }
+        if (c < nchunk) orow[c] = quantise_h8(v[i], t);
     }
 }
 #endif  // KMI_PREP_BODIES_H

@@ -132,17 +132,28 @@ class DynamicLinear(torch.nn.Module):
                                                      self.group_size, tiled=tiled)
         return buf, tiled
 
-    @torch.no_grad()
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
-        shape = input.shape
-        K = shape[-1]
-        m = input.numel() // K
+    def _select(self, m):
         if m != self.pre_m:
             self.pre_m = m
             comp = type(self).prof.get_comp_type(self.shape, m)
             if self.comp_type is not None and comp != self.comp_type:
                 self.switch_count += 1
             self.comp_type = comp
+        return self.comp_type
+
+    @torch.no_grad()
+    def forward(self, input) -> torch.Tensor:
+        shape = input.shape
+        K = shape[-1]
+        m = input.numel() // K
+        self._select(m)
+        if not isinstance(input, torch.Tensor):              # a MatchedActivation from the operator in front
+            if self.comp_type == _W8A8 and input.int_x is not None:
+                return self._w8a8(None, input.int_x.reshape(-1, K), input.scale_x).reshape(*shape[:-1], -1)
+            if input.f16 is None:
+                raise ValueError("the matched activation holds no fp16 form, but this layer's lane for "
+                                 f"{m} tokens (id {self.comp_type}) needs one")
+            input = input.f16
         if self.comp_type == _W4A16_GEMV and m <= ops.GEMV_MAX_M and ops._tracer is None:
             return self._forward_decode(input, shape, m)
         return self._forward(input.reshape(-1, K), m, self.comp_type).reshape(*shape[:-1], -1)
@@ -164,6 +175,32 @@ class DynamicLinear(torch.nn.Module):
             ops._lib.check(rc)
         return out
 
+    def _w8a8(self, x, int_x, scale_x):
+        """The W8A8 lane on fp16 activations x [m, K], or on activations that arrive quantised (x None)."""
+        N, K = self.shape
+        quantise = int_x is None
+        if quantise:
+            int_x = torch.empty_like(x, dtype=torch.int8)
+            scale_x = torch.empty((x.shape[0],), device=x.device, dtype=torch.float16)
+        m = int_x.shape[0]
+        if self.resident_copies:
+            (w8, tiled), hit = self._converted('i8'), True
+        else:
+            tiled = self._tileable()
+            w8, hit = self._cache().get(self._uid, ('i8', tiled), self.shape, torch.int8, self.qweight.device)
+        if not quantise:
+            if not hit:
+                ops.dequant_interleaved_int4_to_int8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8,
+                                                     self.group_size, tiled=tiled)
+        elif hit:
+            ops.quant_fp16_to_int8(int_x, x, scale_x)
+        else:                                                # conversion and quantisation share one launch
+            ops.prep_w8a8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8, int_x, x, scale_x,
+                          self.group_size, tiled=tiled)
+        out = torch.empty((m, N), device=int_x.device, dtype=torch.float16)
+        ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
+        return out
+
     @torch.no_grad()
     def _forward(self, input: torch.Tensor, batch_token_len, comp_type) -> torch.Tensor:
         N, K = self.shape
@@ -178,20 +215,7 @@ class DynamicLinear(torch.nn.Module):
         elif comp_type in (_W4A16_GEMM, _W4A16_GEMV):
             out = ops.gemm_forward(x, self.qweight, self.scales, self.scaled_zeros, bias=self.bias)
         elif comp_type == _W8A8:
-            int_x = torch.empty_like(x, dtype=torch.int8)
-            scale_x = torch.empty((m,), device=x.device, dtype=torch.float16)
-            if self.resident_copies:
-                (w8, tiled), hit = self._converted('i8'), True
-            else:
-                tiled = self._tileable()
-                w8, hit = self._cache().get(self._uid, ('i8', tiled), self.shape, torch.int8, self.qweight.device)
-            if hit:
-                ops.quant_fp16_to_int8(int_x, x, scale_x)
-            else:                                            # conversion and quantisation share one launch
-                ops.prep_w8a8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8, int_x, x, scale_x,
-                              self.group_size, tiled=tiled)
-            out = torch.empty((m, N), device=x.device, dtype=torch.float16)
-            ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
+            out = self._w8a8(x, None, None)
         elif comp_type in (_W8A16_GEMM, _W8A16_GEMV):
             w8, _ = self._converted('i8', tiled=False)       # this lane widens int8 in registers: row-major source
             out = ops.w8a16_gemm_forward(x, w8, self.scales_1, N, bias=self.bias)

@@ -95,6 +95,35 @@ def quant_fp16_to_int8(out, input, scale):
           M, K, _stream())
 
 
+def rmsnorm_quant(x, gamma, eps, residual=None, want_f16=True, want_i8=True):
+    """RMSNorm of x (of x + residual when given) emitting the activation formats asked for, in one launch.
+
+    x, residual fp16 [..., K]; gamma fp16 [K].  Returns (y, int_x, scale_x, h): y fp16 like x or None; int_x int8
+    like x and scale_x fp16 [tokens], or None, None; h = fp16(x + residual), the updated residual stream, or None
+    without a residual.  int_x / scale_x equal quant_fp16_to_int8 applied to y bit for bit."""
+    _need(x, torch.float16, "x"); _need(gamma, torch.float16, "gamma")
+    if not (want_f16 or want_i8):
+        raise ValueError("rmsnorm_quant: at least one output format is needed")
+    K = x.shape[-1]
+    if gamma.numel() != K:
+        raise ValueError(f"rmsnorm_quant: gamma has {gamma.numel()} entries, x {K} columns")
+    M = x.numel() // K if K else 0
+    h = None
+    if residual is not None:
+        _need(residual, torch.float16, "residual")
+        if residual.shape != x.shape:
+            raise ValueError("rmsnorm_quant: residual and x differ in shape")
+        h = torch.empty_like(x)
+    y = torch.empty_like(x) if want_f16 else None
+    int_x = torch.empty_like(x, dtype=torch.int8) if want_i8 else None
+    scale_x = torch.empty((M,), dtype=torch.float16, device=x.device) if want_i8 else None
+    if M == 0:
+        return y, int_x, scale_x, h
+    _call("rmsnorm_quant_act", M, 0, K, _lib.load().kmi_rmsnorm_quant_act, _ptr(int_x), _ptr(scale_x), _ptr(y), _ptr(h),
+          x.data_ptr(), _ptr(residual), gamma.data_ptr(), float(eps), M, K, _stream())
+    return y, int_x, scale_x, h
+
+
 def prep_w8a8(w8_out, qweight, scale_to8, scaled_zero_to8, int_x, x, scale_x, group_size=GROUP_SIZE, tiled=False):
     """int4 -> int8 weight conversion and per-token activation quantisation in one launch (bit-identical to
     dequant_interleaved_int4_to_int8 followed by quant_fp16_to_int8)."""

@@ -30,6 +30,11 @@ Pinning status (what, other than this file agreeing with itself, fixes each func
                                   demands trans(pack_awq(A)) == pack_w4a8(A) bit for bit (test_trans_layout.py:46-52);
                                   both statements re-typed in tests/test_oracle_layout.py plus the index formula
                                   by brute force.
+  rmsnorm_f16                     parity unpinned by the reference (its modules run the eager PyTorch norm of the
+                                  checkpoint, which is not importable here): pinned by closed-form rows (constant
+                                  magnitude, so the sum, the root and the reciprocal are exact), by torch's own
+                                  CPU ops composed as the eager module composes them, and by the float64 sum
+                                  (at most one fp16 step apart, equal on almost every element).
   LUT                             reference C++ header compiled into oracle/_ref (see Makefile) and
                                   the two shipped table files.
 """
@@ -304,6 +309,62 @@ def quant_act_i8(x):
     p = np.where(np.isnan(p), np.float32(0), p)
     q = np.clip(np.rint(p), -128, 127).astype(np.int8)
     return q, scale.reshape(-1)
+
+
+# ----------------------------------------------------------------------------------------------
+# RMSNorm in front of the quantiser ("activation matching", README.md:23-27)
+# ----------------------------------------------------------------------------------------------
+def rmsnorm_f16(x, gamma, eps, residual=None, exact_sum=False):
+    """The fp16 RMSNorm of the decoder modules the reference quantises (transformers LlamaRMSNorm /
+    Qwen2RMSNorm, which kairos/smooth_scale.py:112-119 addresses as input_layernorm / post_attention_layernorm),
+    every intermediate rounded as the eager module rounds it:
+        h = fp16(x + residual);  var = mean(float(h)^2);  y = gamma * fp16(float(h) * rsqrt(var + eps)).
+    fp16 [M, K] -> (y fp16 [M, K], h fp16 [M, K]).
+
+    The fp32 sum of squares depends on the order of addition.  exact_sum=False follows the order of the HIP
+    kernel (256 threads per token; thread t owns the 8-element chunks t, t+256, ..; per thread in order;
+    butterfly over each 64-lane wave with xor 32, 16, .., 1; then (w0 + w1) + (w2 + w3)), which makes the
+    comparison with the kernel bit-exact.  exact_sum=True sums in float64 (exact for these inputs up to one final rounding) and is
+    the order-free statement the other one is checked against.
+    """
+    h = np.asarray(x, dtype=np.float16)
+    if residual is not None:
+        h = (h + np.asarray(residual, dtype=np.float16)).astype(np.float16)      # numpy adds fp16 with one rounding
+    M, K = h.shape
+    hf = h.astype(np.float32)
+    if exact_sum:
+        total = (hf.astype(np.float64) ** 2).sum(axis=1).astype(np.float32)
+    else:
+        nchunk = K // 8
+        tpt = 256                                                                 # threads per token
+        cpt = (nchunk + tpt - 1) // tpt
+        sq = np.zeros((M, cpt * tpt, 8), dtype=np.float32)
+        sq[:, :nchunk, :] = (hf * hf).reshape(M, nchunk, 8)                       # exact: 22-bit products
+        sq = sq.reshape(M, cpt, tpt, 8)
+        ss = np.zeros((M, tpt), dtype=np.float32)
+        for i in range(cpt):
+            for e in range(8):
+                ss = ss + sq[:, i, :, e]
+        ss = ss.reshape(M, tpt // 64, 64)
+        lanes = np.arange(64)
+        for off in (32, 16, 8, 4, 2, 1):
+            ss = ss + ss[:, :, lanes ^ off]
+        w = ss[:, :, 0]
+        total = (w[:, 0] + w[:, 1]) + (w[:, 2] + w[:, 3])
+    var = total / np.float32(K)
+    with np.errstate(divide="ignore"):
+        r = np.float32(1) / np.sqrt(var + np.float32(eps), dtype=np.float32)
+    t = (hf * r[:, None]).astype(np.float16)
+    y = (np.asarray(gamma, dtype=np.float16).astype(np.float32)[None, :] * t.astype(np.float32)).astype(np.float16)
+    return y, h
+
+
+def rmsnorm_quant_act(x, gamma, eps, residual=None):
+    """rmsnorm_f16 followed by quant_act_i8: what the fused kernel must equal bit for bit.
+    -> (int8 [M, K], scale fp16 [M], y fp16 [M, K], h fp16 [M, K])."""
+    y, h = rmsnorm_f16(x, gamma, eps, residual)
+    q, s = quant_act_i8(y)
+    return q, s, y, h
 
 
 # ----------------------------------------------------------------------------------------------

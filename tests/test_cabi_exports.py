@@ -74,6 +74,15 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_trans_layout_w4a8(None, 16, 32, 64, None) == -1
     assert lib.kmi_trans_layout_w4a8(16, 16, 16, 64, None) == -2 and lib.kmi_trans_layout_w4a8(16, 16, 32, 32, None) == -2
     assert lib.kmi_trans_layout_w4a8(16, 8, 32, 64, None) == -5
+    # norm + quantiser: x and gamma always, at least one output, a scale with the int8 output
+    assert lib.kmi_rmsnorm_quant_act(16, 16, 16, None, None, None, 16, 1e-5, 2, 128, None) == -1
+    assert lib.kmi_rmsnorm_quant_act(None, None, None, None, 16, None, 16, 1e-5, 2, 128, None) == -1
+    assert lib.kmi_rmsnorm_quant_act(16, None, None, None, 16, None, 16, 1e-5, 2, 128, None) == -1
+    assert lib.kmi_rmsnorm_quant_act(None, None, 16, 16, 16, None, 16, 1e-5, 2, 128, None) == -1    # h_out without a residual
+    assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 8, 1e-5, 2, 128, None) == -5
+    assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, 1e-5, 2, 100, None) == -2
+    assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, -1.0, 2, 128, None) == -2
+    assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, 1e-5, 0, 128, None) == 0
     assert lib.kmi_lut_get(None, 3) == -7
 
 
