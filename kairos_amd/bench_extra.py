@@ -5,6 +5,7 @@
     python -m kairos_amd.bench_extra decoder   # random-init Llama-3-8B decoder: TTFT / TPOT / lane switches
     python -m kairos_amd.bench_extra blasref   # the library's int8 / fp16 GEMMs of this image (hipBLASLt via torch) beside this build's
     python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
+    python -m kairos_amd.bench_extra actnorm   # per-token quantiser and fused residual add + RMSNorm + quantiser, GB/s
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -198,6 +199,43 @@ def weightprep(args):
         torch.cuda.empty_cache()
     return {"bench": "weightprep", "rows": rows,
             "algorithmic_bytes": "2*N*K (fp16 in) + N*K/2 (int4 out) + 4*(K/128)*N*2 (tables) + 2*N (channel scales)"}
+
+
+def actnorm(args):
+    """The operators that hand activations to a switched linear, on Llama-3-8B's hidden size: the stand-alone per-token
+    quantiser, and residual add + RMSNorm emitting int8, fp16 or both.  The torch column is the same work as separate
+    PyTorch kernels (add, rms_norm) followed by the stand-alone quantiser."""
+    dev = torch.device("cuda:0")
+    K = 4096
+    gamma = torch.ones(K, dtype=torch.float16, device=dev)
+    rows = []
+    for M in (16, 256, 2048, 4096, 32768):
+        n = max(2, min(8, int(800e6 // (M * K * 4))))
+        xs = [torch.randn(M, K, dtype=torch.float16, device=dev) for _ in range(n)]
+        rs = [torch.randn(M, K, dtype=torch.float16, device=dev) for _ in range(n)]
+        q = torch.empty(M, K, dtype=torch.int8, device=dev)
+        sc = torch.empty(M, dtype=torch.float16, device=dev)
+
+        def torch_chain(i):
+            y = torch.nn.functional.rms_norm(xs[i % n] + rs[i % n], (K,), gamma, 1e-5)
+            ops.quant_fp16_to_int8(q, y, sc)
+        cases = [
+            ("quantiser alone", 3 * M * K + 2 * M, lambda i: ops.quant_fp16_to_int8(q, xs[i % n], sc)),
+            ("norm -> int8", 3 * M * K + 2 * M, lambda i: ops.rmsnorm_quant(xs[i % n], gamma, 1e-5, want_f16=False)),
+            ("norm -> fp16", 4 * M * K, lambda i: ops.rmsnorm_quant(xs[i % n], gamma, 1e-5, want_i8=False)),
+            ("add + norm -> int8", 7 * M * K + 2 * M, lambda i: ops.rmsnorm_quant(xs[i % n], gamma, 1e-5, rs[i % n], want_f16=False)),
+            ("add + norm -> int8 + fp16", 9 * M * K + 2 * M, lambda i: ops.rmsnorm_quant(xs[i % n], gamma, 1e-5, rs[i % n])),
+            ("torch add, rms_norm + quantiser", 7 * M * K + 2 * M, torch_chain),
+        ]
+        for name, nbytes, fn in cases:
+            us = _time(fn, 50)
+            rows.append({"M": M, "K": K, "op": name, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                         "hbm_frac": round(nbytes / us / 1e-6 / HBM, 4)})
+            print(rows[-1], file=sys.stderr, flush=True)
+        del xs, rs
+        torch.cuda.empty_cache()
+    return {"bench": "actnorm", "rows": rows,
+            "algorithmic_bytes": "2*M*K per fp16 tensor read or written, M*K + 2*M for the int8 form (gamma's 2*K not counted)"}
 
 
 # ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
@@ -419,6 +457,7 @@ def main(argv=None):
     sub.add_parser("convert")
     sub.add_parser("weightprep")
     sub.add_parser("blasref")
+    sub.add_parser("actnorm")
     d = sub.add_parser("decoder")
     d.add_argument("--lut", default=None)
     d.add_argument("--layers", type=int, default=32)
@@ -436,7 +475,7 @@ def main(argv=None):
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
     ops.ensure_workspace()
-    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

@@ -270,3 +270,38 @@ def test_apply_scale_keeps_the_fp_function():
     assert torch.allclose(before, after, rtol=1e-4, atol=1e-4)
     with pytest.raises(ValueError):
         apply_scale(model, [[("no_such_op", ["mlp.down_proj"], torch.ones(1, 512))]])
+
+
+def test_matched_norm_asks_its_consumers_for_their_lane():
+    """Host half of activation matching: the formats a norm emits follow the table lookups of its consumers
+    (int8 where a lane is W8A8, fp16 elsewhere, both when consumers disagree); no GPU involved."""
+    import torch
+    from kairos.act_matching import MatchedActivation, MatchedRMSNorm
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.perf_profiler import Profiler
+    shapes = [(256, 512), (384, 512)]
+    prof = Profiler(shapes)
+    for r, name in [(8, 'w4a16_gemv'), (64, 'w4a16_gemm'), (4096, 'w8a8')]:
+        prof.record_best_comp(shapes[0], r, name)
+    for r, name in [(8, 'w4a16_gemv'), (256, 'w4a16_gemm'), (4096, 'w8a8')]:
+        prof.record_best_comp(shapes[1], r, name)
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        lins = [DynamicLinear(512, n, False, 'cpu', 128) for n, _ in shapes]
+        norm = MatchedRMSNorm(torch.ones(512, dtype=torch.float16), 1e-5, lins)
+        assert norm.formats_for(4) == (True, False)
+        assert norm.formats_for(64) == (True, False)
+        assert norm.formats_for(65) == (True, True)
+        assert norm.formats_for(257) == (False, True)
+        assert MatchedRMSNorm(norm.weight, 1e-5, [torch.nn.Linear(512, 8)]).formats_for(300) == (True, False)
+
+        class Norm:                                           # the two attribute names of the decoder families
+            weight, variance_epsilon = norm.weight, 1e-6
+        assert MatchedRMSNorm.from_module(Norm, lins).eps == 1e-6
+        act = MatchedActivation(None, torch.zeros(2, 3, 512, dtype=torch.int8), torch.zeros(6, dtype=torch.float16))
+        assert act.shape == (2, 3, 512) and act.numel() == 2 * 3 * 512
+        with pytest.raises(ValueError):                       # lane for 6 tokens is fp16-fed, the activation is int8 only
+            lins[0](act)
+    finally:
+        DynamicLinear.prof = old
