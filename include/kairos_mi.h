@@ -97,6 +97,15 @@ int kmi_prep_w8a8(void* w8_out, int tiled, const void* qweight, const void* scal
 int kmi_rmsnorm_quant_act(void* a8_out, void* ascale_f16, void* y_f16_out, void* h_f16_out, const void* x_f16,
                           const void* residual_f16, const void* gamma_f16, float eps, int M, int K, void* stream);
 
+/* The operator in front of the down projection, in the format of its lane (same idea as kmi_rmsnorm_quant_act; the
+ * reference runs the checkpoint's eager act_fn(gate) * up and quantises inside _forward, kairos/dynamic_linear.py:150-152).
+ * gate_up_f16 [M, 2*I]: gate in columns 0..I-1, up in columns I..2I-1.  s = fp16(g / (1 + exp(-g))) evaluated in fp32
+ * with the hardware exponential and reciprocal; y = fp16(float(s) * float(u)).  y_f16_out [M, I] (may be NULL) receives
+ * y; a8_out [M, I] / ascale_f16 [M] (may both be NULL) receive kmi_quant_act_i8 of y, bit for bit.  s is within one
+ * fp16 step of the correctly rounded SiLU (y within two).  Needs I%8==0, I<=32768, 16-byte aligned tensors. */
+int kmi_silu_mul_quant_act(void* a8_out, void* ascale_f16, void* y_f16_out, const void* gate_up_f16, int M, int I,
+                           void* stream);
+
 /* ---- offline weight preparation ----------------------------------------------------------------- */
 
 /* fp16 weight [N, K] (row-major) -> the resident format of one linear, in one launch:

@@ -24,6 +24,7 @@ SIGNATURES = {
     "kmi_quant_act_i8": [_P, _P, _P, _I, _I, _P],
     "kmi_prep_w8a8": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P, _I, _P],
     "kmi_rmsnorm_quant_act": [_P, _P, _P, _P, _P, _P, _P, ctypes.c_float, _I, _I, _P],
+    "kmi_silu_mul_quant_act": [_P, _P, _P, _P, _I, _I, _P],
     "kmi_prepare_weight": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "kmi_padded_groups": [_I, _I],
     "kmi_trans_layout_w4a8": [_P, _P, _I, _I, _P],

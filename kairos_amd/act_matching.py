@@ -5,7 +5,8 @@ FP16, the quantization step is simply skipped").
 
 The reference's modules quantise inside `_forward` (kairos/dynamic_linear.py:150-152); here the decoder's RMSNorm
 asks its consumers which lane they will take for this token count and emits fp16, int8 + per-token scales, or
-both, from one read of the hidden state (`kmi_rmsnorm_quant_act`).  A `MatchedActivation` carries the result to
+both, from one read of the hidden state (`kmi_rmsnorm_quant_act`); the SiLU(gate) * up in front of the down
+projection does the same (`kmi_silu_mul_quant_act`).  A `MatchedActivation` carries the result to
 `DynamicLinear.forward`, which skips its own quantiser when the int8 form is already there.
 """
 import torch
@@ -24,6 +25,18 @@ class MatchedActivation:
 
     def numel(self):
         return (self.f16 if self.f16 is not None else self.int_x).numel()
+
+
+def _formats_for(consumers, m):
+    """(want_f16, want_i8) for m tokens: int8 if a consumer's lane is W8A8, fp16 if one is anything else."""
+    want_f16 = want_i8 = False
+    for lin in consumers:
+        comp = type(lin).prof.get_comp_type(lin.shape, m) if isinstance(lin, DynamicLinear) else None
+        if comp == _W8A8:
+            want_i8 = True
+        else:
+            want_f16 = True
+    return want_f16, want_i8
 
 
 class MatchedRMSNorm(torch.nn.Module):
@@ -48,15 +61,7 @@ class MatchedRMSNorm(torch.nn.Module):
         return cls(norm.weight, eps, consumers)
 
     def formats_for(self, m):
-        """(want_f16, want_i8) for m tokens: int8 if a consumer's lane is W8A8, fp16 if one is anything else."""
-        want_f16 = want_i8 = False
-        for lin in self.consumers:
-            comp = type(lin).prof.get_comp_type(lin.shape, m) if isinstance(lin, DynamicLinear) else None
-            if comp == _W8A8:
-                want_i8 = True
-            else:
-                want_f16 = True
-        return want_f16, want_i8
+        return _formats_for(self.consumers, m)
 
     @torch.no_grad()
     def forward(self, x, residual=None):
@@ -64,3 +69,20 @@ class MatchedRMSNorm(torch.nn.Module):
         want_f16, want_i8 = self.formats_for(x.numel() // K)
         y, int_x, scale_x, h = ops.rmsnorm_quant(x, self.weight, self.eps, residual, want_f16, want_i8)
         return MatchedActivation(y, int_x, scale_x), h
+
+
+class MatchedSiluMul(torch.nn.Module):
+    """SiLU(gate) * up in front of the down projection, in the format of that projection's lane.
+    forward(gate_up [..., 2*I], gate first) -> MatchedActivation [..., I]."""
+
+    def __init__(self, consumers):
+        super().__init__()
+        self.consumers = list(consumers)
+
+    def formats_for(self, m):
+        return _formats_for(self.consumers, m)
+
+    @torch.no_grad()
+    def forward(self, gate_up):
+        want_f16, want_i8 = self.formats_for(gate_up.numel() // gate_up.shape[-1])
+        return MatchedActivation(*ops.silu_mul_quant(gate_up, want_f16, want_i8))

@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from . import ops
-from .act_matching import MatchedRMSNorm
+from .act_matching import MatchedRMSNorm, MatchedSiluMul
 from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
 from .perf_profiler import Profiler
 from .temp_cache import TempCache
@@ -202,8 +202,8 @@ def weightprep(args):
 
 
 def actnorm(args):
-    """The operators that hand activations to a switched linear, on Llama-3-8B's hidden size: the stand-alone per-token
-    quantiser, and residual add + RMSNorm emitting int8, fp16 or both.  The torch column is the same work as separate
+    """The operators that hand activations to a switched linear, on Llama-3-8B's sizes: the stand-alone per-token
+    quantiser, residual add + RMSNorm emitting int8, fp16 or both (K = 4096), and SiLU(gate) * up (I = 14336).  The torch column is the same work as separate
     PyTorch kernels (add, rms_norm) followed by the stand-alone quantiser."""
     dev = torch.device("cuda:0")
     K = 4096
@@ -233,6 +233,26 @@ def actnorm(args):
                          "hbm_frac": round(nbytes / us / 1e-6 / HBM, 4)})
             print(rows[-1], file=sys.stderr, flush=True)
         del xs, rs
+        torch.cuda.empty_cache()
+    I = 14336
+    for M in (16, 2048, 32768):
+        n = max(2, min(8, int(1600e6 // (M * I * 4))))
+        gus = [torch.randn(M, 2 * I, dtype=torch.float16, device=dev) for _ in range(n)]
+        q = torch.empty(M, I, dtype=torch.int8, device=dev)
+        sc = torch.empty(M, dtype=torch.float16, device=dev)
+
+        def torch_silu(i):
+            g, u = gus[i % n].chunk(2, dim=-1)
+            ops.quant_fp16_to_int8(q, torch.nn.functional.silu(g) * u, sc)
+        for name, nbytes, fn in [
+                ("silu * up -> int8", 5 * M * I + 2 * M, lambda i: ops.silu_mul_quant(gus[i % n], want_f16=False)),
+                ("silu * up -> fp16", 6 * M * I, lambda i: ops.silu_mul_quant(gus[i % n], want_i8=False)),
+                ("torch silu, mul + quantiser", 5 * M * I + 2 * M, torch_silu)]:
+            us = _time(fn, 30)
+            rows.append({"M": M, "K": I, "op": name, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                         "hbm_frac": round(nbytes / us / 1e-6 / HBM, 4)})
+            print(rows[-1], file=sys.stderr, flush=True)
+        del gus
         torch.cuda.empty_cache()
     return {"bench": "actnorm", "rows": rows,
             "algorithmic_bytes": "2*M*K per fp16 tensor read or written, M*K + 2*M for the int8 form (gamma's 2*K not counted)"}
@@ -277,6 +297,7 @@ class _Layer(torch.nn.Module):
         if matched:
             self.n1 = MatchedRMSNorm(self.n1.weight, 1e-5, [self.qkv])
             self.n2 = MatchedRMSNorm(self.n2.weight, 1e-5, [self.gate_up])
+            self.act = MatchedSiluMul([self.down])
         self.matched = matched
         self.k_cache = self.v_cache = None
 
@@ -303,7 +324,10 @@ class _Layer(torch.nn.Module):
     def _mlp(self, x, a):
         B, S, _ = x.shape
         y, x = self._norm(self.n2, x, self.o(a.transpose(1, 2).reshape(B, S, -1)))
-        g, u = self.gate_up(y).chunk(2, dim=-1)
+        gu = self.gate_up(y)
+        if self.matched:
+            return x, self.down(self.act(gu))
+        g, u = gu.chunk(2, dim=-1)
         return x, self.down(torch.nn.functional.silu(g) * u)
 
     def prefill(self, x, delta):
@@ -444,8 +468,8 @@ def decoder(args):
         torch.cuda.empty_cache()
     return {"bench": "decoder", "layers": nl, "prompt": args.prompt, "new_tokens": args.new_tokens,
             "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention in PyTorch over a static KV cache, "
-                    + ("norms in PyTorch" if args.torch_norm else "residual add + RMSNorm + activation format of the next lane in "
-                       "one kernel (kmi_rmsnorm_quant_act)") + ", greedy decoding",
+                    + ("norms and SiLU * up in PyTorch" if args.torch_norm else "residual add + RMSNorm, and SiLU * up, each with the "
+                       "activation format of the next lane in one kernel (kmi_rmsnorm_quant_act, kmi_silu_mul_quant_act)") + ", greedy decoding",
             "norms": "torch" if args.torch_norm else "matched",
             "peak_hbm_gb": round(torch.cuda.max_memory_allocated() / 1e9, 2), "rows": results}
 
@@ -466,7 +490,7 @@ def main(argv=None):
     d.add_argument("--ttft-times", type=int, default=3)
     d.add_argument("--batches", type=int, nargs="+", default=[2, 4, 8, 16, 32])
     d.add_argument("--eager-decode", action="store_true", help="step token by token from Python instead of replaying a HIP graph")
-    d.add_argument("--torch-norm", action="store_true", help="PyTorch residual adds and RMSNorms instead of the fused matched norm")
+    d.add_argument("--torch-norm", action="store_true", help="PyTorch residual adds, RMSNorms and SiLU * up instead of the fused matched operators")
     d.add_argument("--check-tokens", type=int, default=8, help="tokens generated both eagerly and by replay, compared")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():

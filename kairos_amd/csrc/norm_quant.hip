@@ -1,3 +1,5 @@
+// The operators in front of a switched linear, fused with the per-token activation quantiser.  Second half of the
+// file: SiLU(gate) * up in front of the down projection.  First half:
 // RMSNorm (optionally behind a residual add) fused with the per-token activation quantiser: the operator in front
 // of a switched linear layer emits the activation format its consumer's lane needs -- fp16, int8 + per-token scale,
 // or both -- from ONE read of the hidden state.  One workgroup per token; the row lives in registers between the
@@ -134,5 +136,89 @@ extern "C" int kmi_rmsnorm_quant_act(void* a8_out, void* ascale_f16, void* y_f16
     else if (cpt <= 8) KMI_NORM_LAUNCH(8);
     else KMI_NORM_LAUNCH(16);
 #undef KMI_NORM_LAUNCH
+    return kmi_check_launch(fn);
+}
+
+// ---- SiLU(gate) * up in front of the down projection --------------------------------------------------------------
+// gate_up [M, 2*I] fp16 (gate in columns 0..I-1, up in I..2I-1, the output of the fused gate/up linear):
+//   s = fp16(g / (1 + exp(-g)))  evaluated in fp32;   y = fp16(float(s) * float(u));   int8 = quantiser of y.
+// The exponential and the reciprocal are the hardware approximations (about 1e-7 relative, four thousand times finer
+// than the fp16 rounding that follows), so s can differ from a correctly rounded evaluation by one fp16 step (y by two)
+// on roughly one element in a thousand; the int8 output is exactly the quantiser applied to the y this kernel produces.
+// One workgroup per token, the row of products stays in registers between the two phases.
+// Algorithmic traffic: 4*M*I bytes in, M*I + 2*M (int8) and / or 2*M*I (fp16) out.
+template <int CPT>
+__global__ __launch_bounds__(256) void silu_mul_quant_kernel(int8_t* __restrict__ a8, half_t* __restrict__ ascale,
+                                                             half_t* __restrict__ y_out,
+                                                             const half_t* __restrict__ gate_up, int I) {
+    const int token = blockIdx.x;
+    const int nchunk = I >> 3;
+    const h8_t* gr = reinterpret_cast<const h8_t*>(gate_up + (long)token * 2 * I);
+    const h8_t* ur = reinterpret_cast<const h8_t*>(gate_up + (long)token * 2 * I + I);
+    __shared__ float red_amax[4];
+
+    h8_t v[CPT], u[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < nchunk) { v[i] = gr[c]; u[i] = ur[c]; }
+    }
+    h2_t am2 = {(half_t)0.0f, (half_t)0.0f};
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < nchunk) {
+            h8_t sg;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float g = (float)v[i][e];
+                sg[e] = (half_t)(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
+            }
+            v[i] = sg * u[i];                                  // fp16 products: the rounding of the exact product
+            am2 = amax_h8(am2, v[i]);
+            if (y_out) reinterpret_cast<h8_t*>(y_out + (long)token * I)[c] = v[i];
+        }
+    }
+    if (!a8) return;                                           // uniform over the grid
+
+    float amax = wave_max(fmaxf((float)am2[0], (float)am2[1]));
+    if ((threadIdx.x & 63) == 0) red_amax[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red_amax[0], red_amax[1]), fmaxf(red_amax[2], red_amax[3]));
+    if (threadIdx.x == 0) ascale[token] = (half_t)(amax / 127.0f);
+    const float t = 127.0f / amax;                             // IEEE division; +inf for an all-zero token
+    u2_t* orow = reinterpret_cast<u2_t*>(a8 + (long)token * I);
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < nchunk) orow[c] = quantise_h8(v[i], t);
+    }
+}
+
+extern "C" int kmi_silu_mul_quant_act(void* a8_out, void* ascale_f16, void* y_f16_out, const void* gate_up_f16, int M,
+                                      int I, void* stream) {
+    const char* fn = "kmi_silu_mul_quant_act";
+    if (!gate_up_f16) return kmi_set_error(KMI_E_NULL, "%s: gate_up must not be NULL", fn);
+    if (!a8_out && !y_f16_out) return kmi_set_error(KMI_E_NULL, "%s: at least one of a8_out, y_f16_out is needed", fn);
+    if (a8_out && !ascale_f16) return kmi_set_error(KMI_E_NULL, "%s: a8_out needs ascale_f16", fn);
+    if (!kmi_aligned16(a8_out) || !kmi_aligned16(y_f16_out) || !kmi_aligned16(gate_up_f16))
+        return kmi_set_error(KMI_E_ALIGN, "%s: every tensor must be 16-byte aligned", fn);
+    if (M < 0 || I <= 0 || (I & 7) || I > 32768)
+        return kmi_set_error(KMI_E_SHAPE, "%s: need M>=0, I%%8==0, I<=32768 (M=%d I=%d)", fn, M, I);
+    if (M == 0) return KMI_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int8_t* a8 = static_cast<int8_t*>(a8_out);
+    half_t* as = static_cast<half_t*>(ascale_f16);
+    half_t* y = static_cast<half_t*>(y_f16_out);
+    const half_t* gu = static_cast<const half_t*>(gate_up_f16);
+    const int cpt = ((I >> 3) + 255) / 256;
+    const dim3 grid(M), block(256);
+#define KMI_SILU_LAUNCH(C) hipLaunchKernelGGL(silu_mul_quant_kernel<C>, grid, block, 0, st, a8, as, y, gu, I)
+    if (cpt <= 1) KMI_SILU_LAUNCH(1);
+    else if (cpt <= 2) KMI_SILU_LAUNCH(2);
+    else if (cpt <= 4) KMI_SILU_LAUNCH(4);
+    else if (cpt <= 8) KMI_SILU_LAUNCH(8);
+    else KMI_SILU_LAUNCH(16);
+#undef KMI_SILU_LAUNCH
     return kmi_check_launch(fn);
 }

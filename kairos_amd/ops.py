@@ -124,6 +124,28 @@ def rmsnorm_quant(x, gamma, eps, residual=None, want_f16=True, want_i8=True):
     return y, int_x, scale_x, h
 
 
+def silu_mul_quant(gate_up, want_f16=True, want_i8=True):
+    """SiLU(gate) * up of a fused gate/up output [..., 2*I] (gate first), in the formats asked for, in one launch.
+    Returns (y fp16 [..., I] or None, int_x int8 [..., I] or None, scale_x fp16 [tokens] or None); int_x / scale_x equal
+    quant_fp16_to_int8 applied to y bit for bit."""
+    _need(gate_up, torch.float16, "gate_up")
+    if not (want_f16 or want_i8):
+        raise ValueError("silu_mul_quant: at least one output format is needed")
+    if gate_up.shape[-1] % 2:
+        raise ValueError("silu_mul_quant: the last dimension holds gate and up, it must be even")
+    I = gate_up.shape[-1] // 2
+    M = gate_up.numel() // (2 * I) if I else 0
+    shape = gate_up.shape[:-1] + (I,)
+    y = torch.empty(shape, dtype=torch.float16, device=gate_up.device) if want_f16 else None
+    int_x = torch.empty(shape, dtype=torch.int8, device=gate_up.device) if want_i8 else None
+    scale_x = torch.empty((M,), dtype=torch.float16, device=gate_up.device) if want_i8 else None
+    if M == 0:
+        return y, int_x, scale_x
+    _call("silu_mul_quant_act", M, 0, I, _lib.load().kmi_silu_mul_quant_act, _ptr(int_x), _ptr(scale_x), _ptr(y),
+          gate_up.data_ptr(), M, I, _stream())
+    return y, int_x, scale_x
+
+
 def prep_w8a8(w8_out, qweight, scale_to8, scaled_zero_to8, int_x, x, scale_x, group_size=GROUP_SIZE, tiled=False):
     """int4 -> int8 weight conversion and per-token activation quantisation in one launch (bit-identical to
     dequant_interleaved_int4_to_int8 followed by quant_fp16_to_int8)."""

@@ -35,6 +35,10 @@ Pinning status (what, other than this file agreeing with itself, fixes each func
                                   magnitude, so the sum, the root and the reciprocal are exact), by torch's own
                                   CPU ops composed as the eager module composes them, and by the float64 sum
                                   (at most one fp16 step apart, equal on almost every element).
+  silu_mul_f16                    parity unpinned by the reference (eager activation of the checkpoint's module);
+                                  pinned by torch's CPU silu and multiply (one fp16 step: the exponential is not
+                                  correctly rounded in any of the libraries), exact points (0, large |g|) and the
+                                  identity silu(g) - silu(-g) = g.
   LUT                             reference C++ header compiled into oracle/_ref (see Makefile) and
                                   the two shipped table files.
 """
@@ -365,6 +369,21 @@ def rmsnorm_quant_act(x, gamma, eps, residual=None):
     y, h = rmsnorm_f16(x, gamma, eps, residual)
     q, s = quant_act_i8(y)
     return q, s, y, h
+
+
+def silu_mul_f16(gate_up):
+    """The eager fp16 MLP activation in front of the down projection (transformers LlamaMLP / Qwen2MLP:
+    act_fn(gate_proj(x)) * up_proj(x) with act_fn = SiLU), on a fused [M, 2*I] input, gate first:
+        s = fp16(g / (1 + exp(-g))) evaluated in fp32;  y = fp16(float(s) * float(u)).
+    The exponential is not correctly rounded anywhere (numpy, torch and the GPU each have their own), so
+    comparisons against this function allow one fp16 step; everything behind y is exact again."""
+    gu = np.asarray(gate_up, dtype=np.float16)
+    I = gu.shape[1] // 2
+    g = gu[:, :I].astype(np.float32)
+    u = gu[:, I:].astype(np.float32)
+    with np.errstate(over="ignore"):
+        s = (g / (np.float32(1) + np.exp(-g, dtype=np.float32))).astype(np.float16)
+    return (s.astype(np.float32) * u).astype(np.float16)
 
 
 # ----------------------------------------------------------------------------------------------

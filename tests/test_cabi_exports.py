@@ -83,6 +83,12 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, 1e-5, 2, 100, None) == -2
     assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, -1.0, 2, 128, None) == -2
     assert lib.kmi_rmsnorm_quant_act(None, None, 16, None, 16, None, 16, 1e-5, 0, 128, None) == 0
+    assert lib.kmi_silu_mul_quant_act(16, 16, 16, None, 2, 128, None) == -1
+    assert lib.kmi_silu_mul_quant_act(None, None, None, 16, 2, 128, None) == -1
+    assert lib.kmi_silu_mul_quant_act(16, None, None, 16, 2, 128, None) == -1
+    assert lib.kmi_silu_mul_quant_act(None, None, 8, 16, 2, 128, None) == -5
+    assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 2, 100, None) == -2
+    assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 0, 128, None) == 0
     assert lib.kmi_lut_get(None, 3) == -7
 
 

@@ -142,3 +142,75 @@ def test_dynamic_linear_consumes_matched_activations(ops):
             lins[0](only_i8)
     finally:
         DynamicLinear.prof = old
+
+
+@pytest.mark.parametrize("M,I", [(1, 128), (7, 1000), (33, 14336), (3, 18944), (2, 32768)])
+def test_silu_mul_quant_against_oracle(ops, M, I):
+    """SiLU within one fp16 step of the oracle (the exponential is an approximation on both sides), hence y within
+    two, equal on > 99 % of the elements; the int8 / scale outputs are exactly the quantiser applied to the y the kernel produced, whichever
+    outputs were asked for."""
+    rng = np.random.default_rng(M + I)
+    gu = (rng.standard_normal((M, 2 * I)) * 2.5).astype(np.float16)
+    gu[:, ::97] *= 8
+    y, q, s = ops.silu_mul_quant(dev(gu))
+    want = O.silu_mul_f16(gu)
+    a, b = y.cpu().numpy().view(np.uint16).astype(np.int32), want.view(np.uint16).astype(np.int32)
+    line = lambda u: np.where(u & 0x8000, -(u & 0x7FFF), u)
+    d = np.abs(line(a) - line(b))
+    assert d.max() <= 2 and (d == 0).mean() > 0.99, (d.max(), (d == 0).mean())
+    q_ref, s_ref = O.quant_act_i8(y.cpu().numpy())
+    assert np.array_equal(q.cpu().numpy(), q_ref) and np.array_equal(bits(s), s_ref.view(np.uint16))
+    y2, none_q, none_s = ops.silu_mul_quant(dev(gu), want_i8=False)
+    assert none_q is None and none_s is None and torch.equal(y2.view(torch.int16), y.view(torch.int16))
+    none_y, q2, s2 = ops.silu_mul_quant(dev(gu), want_f16=False)
+    assert none_y is None and torch.equal(q2, q) and torch.equal(s2.view(torch.int16), s.view(torch.int16))
+
+
+def test_silu_mul_quant_full_size_and_exact_points(ops):
+    M, I = 4096, 14336
+    g = torch.Generator(device="cuda").manual_seed(3)
+    gu = torch.randn((M, 2 * I), generator=g, device="cuda", dtype=torch.float16) * 2
+    y, q, s = ops.silu_mul_quant(gu)
+    q2, s2 = torch.empty_like(q), torch.empty_like(s)
+    ops.quant_fp16_to_int8(q2, y, s2)
+    assert torch.equal(q, q2) and torch.equal(s.view(torch.int16), s2.view(torch.int16))
+    ref = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]              # the eager module on the same device
+    assert float((y.float() - ref.float()).abs().max()) <= float(ref.abs().max()) * 2.0 ** -10
+    rows = torch.tensor([0, 1, M // 2, M - 1], device="cuda")
+    want = O.silu_mul_f16(gu[rows].cpu().numpy())
+    got = y[rows].cpu().numpy()
+    assert (got.view(np.uint16) == want.view(np.uint16)).mean() > 0.99
+    # exact points: silu(0) * u = 0, silu(g) = g for g >= 20, an all-zero token quantises to zeros with scale 0
+    pts = torch.tensor([[0.0, 20.0, 64.0, 1000.0] + [0.0] * 4 + [3.0, 0.5, -2.0, 1.0] + [0.0] * 4,
+                        [0.0] * 16], dtype=torch.float16, device="cuda")
+    y, q, s = ops.silu_mul_quant(pts)
+    assert y[0, :4].tolist() == [0.0, 10.0, -128.0, 1000.0] and not y[1].any() and not q[1].any() and float(s[1]) == 0.0
+    with pytest.raises(ValueError):
+        ops.silu_mul_quant(torch.zeros(2, 129, dtype=torch.float16, device="cuda"))
+
+
+def test_matched_silu_mul_feeds_the_down_projection(ops):
+    from kairos.act_matching import MatchedSiluMul
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.perf_profiler import Profiler
+    I, N = 1024, 256
+    prof = Profiler([(N, I)])
+    for r, name in [(8, 'w4a16_gemv'), (64, 'w4a16_gemm'), (4096, 'w8a8')]:
+        prof.record_best_comp((N, I), r, name)
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        lin = torch.nn.Linear(I, N, bias=False, dtype=torch.float16)
+        with torch.no_grad():
+            lin.weight.copy_(torch.from_numpy(O.synth_weights(N, I, seed=31)))
+        down = DynamicLinear.from_module(lin.cuda(), 'cuda')
+        act_fn = MatchedSiluMul([down])
+        for M, formats in [(4, (True, False)), (40, (True, False)), (200, (False, True))]:
+            assert act_fn.formats_for(M) == formats
+            gu = torch.randn((1, M, 2 * I), dtype=torch.float16, device="cuda")
+            act = act_fn(gu)
+            assert act.shape == (1, M, I) and (act.f16 is not None, act.int_x is not None) == formats
+            y = ops.silu_mul_quant(gu, want_i8=False)[0]
+            assert torch.equal(down(act).view(torch.int16), down(y).view(torch.int16))
+    finally:
+        DynamicLinear.prof = old

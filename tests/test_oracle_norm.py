@@ -87,3 +87,27 @@ def test_quantised_form_is_the_quantiser_on_the_norm_output():
     zero = np.zeros((2, 512), dtype=np.float16)                # an all-zero token: zeros and scale 0
     q0, s0, y0, _ = O.rmsnorm_quant_act(zero, gamma, 1e-5)
     assert not q0.any() and not s0.any() and not y0.any()
+
+
+def test_silu_mul_against_torch_cpu_and_exact_points():
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(7)
+    gu = (rng.standard_normal((64, 2 * 512)) * 3).astype(np.float16)
+    y = O.silu_mul_f16(gu)
+    t = torch.from_numpy(gu)
+    ref = (torch.nn.functional.silu(t[:, :512]) * t[:, 512:]).numpy()
+    d = ulp_distance(y, ref)                                  # one step of s can become two of the product
+    assert d.max() <= 2 and (d == 0).mean() > 0.99
+    # exact points: silu(0) = 0; for g >= 20, exp(-g) < 2^-28 so silu(g) = g in fp32; for g <= -20 the result is
+    # below the smallest fp16 subnormal times ... and rounds to -0
+    g = np.array([[0.0, 20.0, 64.0, 1000.0, -30.0, -1000.0]], dtype=np.float16)
+    u = np.array([[3.0, 0.5, -2.0, 1.0, 1.0, 1.0]], dtype=np.float16)
+    out = O.silu_mul_f16(np.concatenate([g, u], axis=1))
+    assert np.array_equal(out[0, :4], np.array([0.0, 10.0, -128.0, 1000.0], dtype=np.float16))
+    assert abs(float(out[0, 4])) < 1e-6 and out[0, 5] == 0
+    # silu(g) - silu(-g) = g: with u = 1 the two halves of a symmetric input differ by g up to the two roundings
+    g = (rng.standard_normal((4, 256)) * 4).astype(np.float16)
+    one = np.ones_like(g)
+    a = O.silu_mul_f16(np.concatenate([g, one], axis=1)).astype(np.float64)
+    b = O.silu_mul_f16(np.concatenate([-g, one], axis=1)).astype(np.float64)
+    assert np.all(np.abs((a - b) - g.astype(np.float64)) <= 2.0 ** -10 * np.maximum(np.abs(g.astype(np.float64)), 2.0 ** -4))
