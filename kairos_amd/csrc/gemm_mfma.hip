@@ -989,9 +989,6 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
         else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);      \
         else KMI_STAGE_BARRIER(0);                                         \
     } while (0)
-#ifdef KMI_DBG_TIMING
-    const uint64_t dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = wall_clock64();
-#endif
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t) issue_stage(t);
     static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
@@ -1019,23 +1016,10 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
     // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 #undef KMI_STAGE_BARRIER
-#ifdef KMI_DBG_TIMING
-    const uint64_t dbg_c1 = __builtin_readcyclecounter(), dbg_r1 = wall_clock64();
-#endif
 
     if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
     else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
-#ifdef KMI_DBG_TIMING
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (p.splits == 1 && p.partial && tid == 0) {
-        uint64_t* d = static_cast<uint64_t*>(p.partial) + (size_t)blockIdx.x * 8;
-        d[0] = dbg_c0; d[1] = dbg_r0; d[2] = dbg_c1; d[3] = dbg_r1;
-        d[4] = __builtin_readcyclecounter(); d[5] = wall_clock64();
-        uint32_t xcc; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        d[6] = xcc; d[7] = blockIdx.x;
-    }
-#endif
 #endif
 }
 
@@ -1103,9 +1087,6 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, in
     const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
     a.splits = whole ? pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units) : 1;
     a.partial = a.splits > 1 ? g_workspace : nullptr;
-#ifdef KMI_DBG_TIMING
-    a.partial = g_workspace;
-#endif
     const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
