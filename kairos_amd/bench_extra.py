@@ -283,6 +283,38 @@ def _rope(x, cs):
     return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
 
 
+class _KernelTimes:
+    """Kernel tracer for ops.set_tracer: device-event brackets around every library launch, summed by kernel name."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def begin(self, name, M, N, K):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self._cur = (name, M, N, K, ev)
+
+    def end(self):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.pairs.append(self._cur + (ev,))
+
+    def seconds(self):
+        """-> (conversion seconds, seconds of every library kernel).  A fused preparation launch counts by the
+        conversion's share of its algorithmic bytes."""
+        torch.cuda.synchronize()
+        conv = total = 0.0
+        for name, M, N, K, e0, e1 in self.pairs:
+            t = e0.elapsed_time(e1) * 1e-3
+            total += t
+            if name.startswith("cvt_i4_to"):
+                conv += t
+            elif name == "prep_w8a8":
+                cb = N * K // 2 + 4 * (K // G) * N + N * K
+                conv += t * cb / (cb + 3 * M * K + 2 * M)
+        return conv, total
+
+
 class _Layer(torch.nn.Module):
     """Pre-norm decoder layer over a static KV cache [B, kv_heads, T_max, d]: prefill fills positions 0..S-1, a
     decode step writes position `pos` (a device tensor, so the step is capturable) and attends under a mask.
@@ -453,8 +485,26 @@ def decoder(args):
         total = time.perf_counter() - t0
         tpot = (total - ttft) / max(1, args.new_tokens - 1)
         sw = [sum(getattr(L, n).switch_count for L in layers) / nl for n in ("qkv", "o", "gate_up", "down")]
+        # conversion overhead of the run: conversions happen where a lane needs a converted weight, i.e. in the prefill
+        # of this table (one traced prefill) and, for a decode lane that converts, in every step (one traced eager step)
+        kt = _KernelTimes()
+        ops.set_tracer(kt)
+        try:
+            first = prefill(ids)
+            conv_prefill, lib_prefill = kt.seconds()
+            kt.pairs = []
+            start(first)
+            step()
+            conv_step, lib_step = kt.seconds()
+        finally:
+            ops.set_tracer(None)
+        conv_run = conv_prefill + conv_step * (args.new_tokens - 1)
         results.append({"batch": B, "ttft_ms": round(ttft * 1e3, 2), "tpot_ms": round(tpot * 1e3, 3),
                         "tokens_per_s": round(B * args.new_tokens / total, 1),
+                        "conversion_share_of_run": round(conv_run / total, 5),
+                        "conversion_share_of_library_kernel_time": round(
+                            conv_run / (lib_prefill + lib_step * (args.new_tokens - 1)), 5),
+                        "conversion_share_of_prefill_library_kernel_time": round(conv_prefill / lib_prefill, 4),
                         "decode": "eager" if graph is None else f"HIP-graph replay, first {args.check_tokens} tokens equal to eager",
                         "switches_per_layer_eager_calls": {"qkv": sw[0], "o_proj": sw[1], "gate_up": sw[2], "down": sw[3]},
                         "prefill_lane": {n: names[prof.get_comp_type(s, B * args.prompt)]
