@@ -57,8 +57,9 @@ def _time(fn, n):
 
 def _layer(N, K, copies, dev):
     """One prepared linear, `copies` times in distinct memory (the values do not matter for timing)."""
-    prep = ops.prepare_weight(_weights(min(N, 1024), K).to(dev))
-    reps = N // min(N, 1024)
+    rows = math.gcd(N, 1024)                       # a slice that tiles N exactly (4608 = 9 x 512, 3584 = 7 x 512)
+    prep = ops.prepare_weight(_weights(rows, K).to(dev))
+    reps = N // rows
     full = {"qweight": prep["qweight"].repeat(reps, 1), "scales_1": prep["scales_1"].repeat(reps)}
     for k in ("scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8"):
         full[k] = prep[k].repeat(1, reps)
@@ -67,6 +68,7 @@ def _layer(N, K, copies, dev):
         dl = DynamicLinear(K, N, False, dev, 128)
         for k, v in full.items():
             setattr(dl, k, v.clone().contiguous())
+        assert dl.qweight.shape == (N // 4, K)
         out.append(dl)
     return out
 

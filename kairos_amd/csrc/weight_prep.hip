@@ -18,8 +18,9 @@
 // d in [1e-10, 1e3]); a zero numerator may come out with the other sign, which the integer conversion and the sum
 // with the zero-point erase.
 //
-// One workgroup per four-row block (the packing unit), one wave per row.  A row is read twice (amax,
-// then quantise); the second read comes from L2.  A 16-byte load is 8 weights of one row; 16 lanes
+// One workgroup per four-row block (the packing unit), one wave per row.  A row of up to 16384 weights is read once
+// and held in registers across the two passes (amax, then quantise); longer rows are read twice.  A 16-byte load is
+// 8 weights of one row; 16 lanes
 // hold one group of 128, 4 lanes one packed 16-byte chunk (32 weights: word t, nibble a, half c holds
 // k = 8a + 2t + c), so lane a of a chunk owns nibble a of all four words and, after an OR across the
 // four lanes, stores word a.
@@ -59,6 +60,9 @@ __device__ __forceinline__ float div_by(float x, float d, float r) {
     return __builtin_fmaf(__builtin_fmaf(-d, q, x), r, q);
 }
 
+// CPL > 0: the row (up to 64 * CPL 16-byte chunks) is loaded once and stays in registers between the two passes;
+// CPL == 0: rows longer than that are read twice, the second time through a one-deep prefetch.
+template <int CPL>
 __global__ __launch_bounds__(256) void prepare_weight_kernel(const half_t* __restrict__ w, int N, int K, int Gp,
                                                              uint32_t* __restrict__ qweight,
                                                              half_t* __restrict__ scales,
@@ -72,15 +76,29 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(const half_t* __res
     const int nch = K >> 3;                      // 16-byte loads per row; a multiple of 16 (K % 128 == 0)
     const int ng = K >> 7;
 
+    constexpr int HELD = CPL > 0 ? CPL : 1;
+    h8_t held[HELD];
     float amax = 0.0f;
-    for (int base = lane; base < nch; base += 256) {       // four independent loads in flight; repeats are harmless
-        h8_t v[4];
+    if constexpr (CPL > 0) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = row[min(base + 64 * u, nch - 1)];
+        for (int i = 0; i < CPL; ++i)
+            if (i * 64 < nch) held[i] = row[min(lane + 64 * i, nch - 1)];             // repeats are harmless
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int i = 0; i < CPL; ++i)
+            if (i * 64 < nch) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)v[u][e]));
+                for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)held[i][e]));
+            }
+    } else {
+        for (int base = lane; base < nch; base += 256) {   // four independent loads in flight; repeats are harmless
+            h8_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = row[min(base + 64 * u, nch - 1)];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)v[u][e]));
+        }
     }
     amax = fmaxf(wave_max(amax), 1e-7f);
     const float s1 = amax / 127.0f;
@@ -89,12 +107,9 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(const half_t* __res
 
     uint32_t* qrow = qweight + (long)quad * (K >> 3) * 4;      // this four-row block: K/8 chunks of 4 words
     const float r1 = refined_rcp(s1);
-    h8_t nxt = row[min(lane, nch - 1)];
-    for (int base = 0; base < nch; base += 64) {
+    auto quantise_chunk = [&](int base, const h8_t& v) {
         const int c = base + lane;
         const bool valid = c < nch;              // uniform over each group of 16 lanes
-        const h8_t v = nxt;
-        nxt = row[min(c + 64, nch - 1)];
         float x[8];
         float hi = -INFINITY, lo = INFINITY;
 #pragma unroll
@@ -137,6 +152,18 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(const half_t* __res
                 szeros[at] = -(half_t)((float)sf * (float)z2h);
             }
         }
+    };
+    if constexpr (CPL > 0) {
+#pragma unroll
+        for (int i = 0; i < CPL; ++i)
+            if (i * 64 < nch) quantise_chunk(i * 64, held[i]);       // wave-uniform
+    } else {
+        h8_t nxt = row[min(lane, nch - 1)];
+        for (int base = 0; base < nch; base += 64) {
+            const h8_t v = nxt;
+            nxt = row[min(base + lane + 64, nch - 1)];
+            quantise_chunk(base, v);
+        }
     }
     for (int g = ng + lane; g < Gp; g += 64) {   // padded table rows are zero
         const long at = (long)g * N + n;
@@ -164,9 +191,16 @@ extern "C" int kmi_prepare_weight(const void* w_f16, int N, int K, int G, void* 
     if (N <= 0 || K <= 0 || (N & 3) || (K & 127))
         return kmi_set_error(KMI_E_SHAPE, "%s: need N%%4==0 and K%%128==0, got N=%d K=%d", fn, N, K);
     const int Gp = ((K / G + 7) / 8) * 8;
-    hipLaunchKernelGGL(prepare_weight_kernel, dim3((unsigned)(N / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const half_t*>(w_f16), N, K, Gp, static_cast<uint32_t*>(qweight),
-                       static_cast<half_t*>(scales), static_cast<half_t*>(scaled_zeros), static_cast<half_t*>(scales_to8),
-                       static_cast<half_t*>(scaled_zeros_to8), static_cast<half_t*>(scales_1));
+    const int cpl = (K / 8 + 63) / 64;              // 16-byte chunks per lane of the wave that owns a row
+#define KMI_PREP_LAUNCH(C)                                                                                              \
+    hipLaunchKernelGGL(prepare_weight_kernel<C>, dim3((unsigned)(N / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), \
+                       static_cast<const half_t*>(w_f16), N, K, Gp, static_cast<uint32_t*>(qweight),                     \
+                       static_cast<half_t*>(scales), static_cast<half_t*>(scaled_zeros), static_cast<half_t*>(scales_to8), \
+                       static_cast<half_t*>(scaled_zeros_to8), static_cast<half_t*>(scales_1))
+    if (cpl <= 8) KMI_PREP_LAUNCH(8);
+    else if (cpl <= 16) KMI_PREP_LAUNCH(16);
+    else if (cpl <= 32) KMI_PREP_LAUNCH(32);
+    else KMI_PREP_LAUNCH(0);
+#undef KMI_PREP_LAUNCH
     return kmi_check_launch(fn);
 }
