@@ -34,7 +34,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
     const int wave = threadIdx.x >> 6;
     const int r16 = lane & 15;
     const int j = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NT);
+    // Workgroup ids are dealt round-robin over the 8 XCDs, each with its own L2.  Neighbouring column strips share
+    // 128-byte lines of the scale tables (a strip of 16*NT columns is 32*NT bytes of a table row), so every XCD takes
+    // a contiguous run of strips: a table line is then fetched by one L2, not by up to four.
+    const int nblk = gridDim.x, xcd = blockIdx.x & 7;
+    const int strip = xcd * (nblk >> 3) + min(xcd, nblk & 7) + (blockIdx.x >> 3);
+    const int n0 = strip * (16 * NT);
     const int ngroups = K >> 7;
     const int kq = K >> 3;                       // 16-byte units per fp16 row of x / per four-row weight block
 
