@@ -201,6 +201,7 @@ static gemv_fn gemv_pick_nt(int nt, int nw) {
         case 1: return gemv_pick_nw<MT, 1>(nw);
         case 2: return gemv_pick_nw<MT, 2>(nw);
         case 4: return gemv_pick_nw<MT, 4>(nw);
+        case 8: return gemv_pick_nw<MT, 8>(nw);
     }
     return nullptr;
 }
@@ -216,7 +217,7 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
 }
 
 // Default split, from sweeps on MI355X over the Llama-3-8B and -70B shapes.
-//   Column tiles per wave (nt): the most of 4, 2, 1 that still leaves about 150 workgroups -- every activation
+//   Column tiles per wave (nt): the most of 4, 2, 1 (8: see the end of the function) that still leaves about 150 workgroups -- every activation
 //   fragment is reused nt times and fewer, longer workgroups stream better (10240 x 8192 at M=16: 14.7 us with
 //   nt=4 and 160 workgroups against 20.8 us with nt=2 and 320) -- except that for M <= 4 a grid that would still be
 //   several rounds of workgroups keeps nt=2 (57344 x 8192 at M=1: 42.8 against 49.7 us).
@@ -231,6 +232,15 @@ static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_o
     if (nt == 1 && (M <= 4 || (M <= 8 && K <= 4096)) && groups >= 16 && gemv_lookup(mt, nt, 16) != nullptr) nw = 16;
     if (mt >= 3 && nt >= 2 && gemv_lookup(mt, nt, 4) != nullptr) nw = 4;
     while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
+    // Eight column tiles for 8..16 tokens on very wide weights: every workgroup reads the whole activation matrix, so
+    // at these M the L2 -> CU traffic for activations equals that for weights; twice the columns per workgroup halves
+    // it (28672 x 4096 at M=16: 16.4 -> 14.6 us; 57344 x 8192: 52.7 -> 45.6 us with four waves).  Only where the
+    // resulting grid still fills the CUs evenly (37888 x 3584 would leave 296 workgroups on 256 CUs: 19.9 -> 22.8 us).
+    const int w8 = (strips + 7) / 8;
+    if (mt == 1 && M >= 8 && w8 >= 200 && ((w8 + 255) / 256) * 256 * 5 <= w8 * 6 && gemv_lookup(1, 8, 8) != nullptr) {
+        nt = 8;
+        nw = w8 > 256 ? 4 : 8;
+    }
     *nt_out = nt;
     *nw_out = nw;
 }

@@ -166,6 +166,21 @@ def test_gemv_every_split(ops, M, nt, nw):
     assert torch.equal(out, again)                          # fixed reduction order
 
 
+@pytest.mark.parametrize("nw", [4, 8])
+@pytest.mark.parametrize("M,N", [(8, 512), (16, 272), (3, 2048)])
+def test_gemv_eight_column_tiles(ops, M, N, nw):
+    """The 128-column workgroup (one row tile only), also with a ragged last strip; more than 16 rows are refused."""
+    K = 1024
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=M)
+    out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128, cfg=(8, nw))
+    assert O.max_abs_rel(host(out), O.gemm_f16(x, p["w16"])) < 2e-3
+    from kairos_amd._lib import KairosMiError
+    with pytest.raises(KairosMiError):
+        ops.gemv_forward(dev(O.synth_acts(17, K, seed=1)), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]),
+                         17, N, K, 128, cfg=(8, nw))
+
+
 def test_gemv_bias_and_ragged_strip(ops):
     N, K, M = 48, 256, 4                                    # N is not a multiple of the 64-column strip
     p = prep(N, K)
