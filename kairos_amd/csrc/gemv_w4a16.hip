@@ -200,7 +200,11 @@ static gemv_fn gemv_pick_nt(int nt, int nw) {
     switch (nt) {
         case 1: return gemv_pick_nw<MT, 1>(nw);
         case 2: return gemv_pick_nw<MT, 2>(nw);
+        case 3: return gemv_pick_nw<MT, 3>(nw);
         case 4: return gemv_pick_nw<MT, 4>(nw);
+        case 5: return gemv_pick_nw<MT, 5>(nw);
+        case 6: return gemv_pick_nw<MT, 6>(nw);
+        case 7: return gemv_pick_nw<MT, 7>(nw);
         case 8: return gemv_pick_nw<MT, 8>(nw);
     }
     return nullptr;
@@ -216,31 +220,37 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
     return nullptr;
 }
 
-// Default split, from sweeps on MI355X over the Llama-3-8B and -70B shapes.
-//   Column tiles per wave (nt): the most of 4, 2, 1 (8: see the end of the function) that still leaves about 150 workgroups -- every activation
-//   fragment is reused nt times and fewer, longer workgroups stream better (10240 x 8192 at M=16: 14.7 us with
-//   nt=4 and 160 workgroups against 20.8 us with nt=2 and 320) -- except that for M <= 4 a grid that would still be
-//   several rounds of workgroups keeps nt=2 (57344 x 8192 at M=1: 42.8 against 49.7 us).
+// Default split, from sweeps on MI355X over the Llama-3-8B / -70B and Qwen2.5-7B shapes.
+//   Column tiles per wave (nt).  All workgroups of these grids are resident at once (up to four per CU), so the
+//   kernel ends when the CU with the most column strips ends: ceil(workgroups / 256) * nt strips.  More tiles per
+//   wave reuse every activation fragment more often (the whole activation matrix is read by every workgroup), less
+//   so at small M; measured times follow  busiest * (1 + c / nt)  with c = 0.6 (M <= 4), 1.0 (M <= 8), 1.7 (M <= 16),
+//   2.5 beyond.  The nt with the smallest estimate wins: 1792 strips (28672 columns) -> 7 tiles, 256 workgroups
+//   (M=16: 14.0 against 16.4 us with 4); 640 strips -> 3 (11.5 against 12.5 us); 2368 -> 5 (14.2 against 15.5);
+//   288 -> 2 (5.1 against 5.9 us with 1).
 //   Waves per workgroup over K (nw): eight; sixteen for a single column tile at the smallest M, where the kernel is
-//   a pure latency chain (4096 x 14336 at M=1: 10.4 against 11.9 us); four from three row tiles on (M > 32).
+//   a pure latency chain (4096 x 14336 at M=1: 10.4 against 11.9 us); four from three row tiles on (M > 32), and for
+//   seven or eight column tiles when more than one workgroup shares a CU (57344 x 8192 at M=16: 45.3 against 48.5 us).
 static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_out) {
     const int strips = (N + 15) / 16, groups = K / 128;
-    int nt = 4;
-    if (M <= 4 && (strips + 3) / 4 > 768) nt = 2;
-    while (nt > 1 && ((strips + nt - 1) / nt < 150 || gemv_lookup(mt, nt, 8) == nullptr)) nt >>= 1;
+    const double c = M <= 4 ? 0.6 : M <= 8 ? 1.0 : M <= 16 ? 1.7 : 2.5;
+    int nt = 1, wgs = strips;
+    double best = 1e30;
+    for (int cand = 1; cand <= 8; ++cand) {
+        if (gemv_lookup(mt, cand, 8) == nullptr) continue;           // row tiles x column tiles <= 8 (registers)
+        const int w = (strips + cand - 1) / cand;
+        const double est = (double)((w + 255) / 256) * (cand + c);    // busiest * (1 + c / nt), busiest = rounds * nt
+        if (est < best - 1e-9) { best = est; nt = cand; wgs = w; }
+    }
+    if (M <= 4 && strips > 3072 && gemv_lookup(mt, 2, 8) != nullptr) {   // many rounds at the smallest M: two tiles stream best
+        nt = 2;                                                         // (128256 x 4096 at M=1: 49.2 against 51.4 us)
+        wgs = (strips + 1) / 2;
+    }
     int nw = 8;
     if (nt == 1 && (M <= 4 || (M <= 8 && K <= 4096)) && groups >= 16 && gemv_lookup(mt, nt, 16) != nullptr) nw = 16;
     if (mt >= 3 && nt >= 2 && gemv_lookup(mt, nt, 4) != nullptr) nw = 4;
+    if (nt >= 7 && wgs > 256 && gemv_lookup(mt, nt, 4) != nullptr) nw = 4;
     while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
-    // Eight column tiles for 8..16 tokens on very wide weights: every workgroup reads the whole activation matrix, so
-    // at these M the L2 -> CU traffic for activations equals that for weights; twice the columns per workgroup halves
-    // it (28672 x 4096 at M=16: 16.4 -> 14.6 us; 57344 x 8192: 52.7 -> 45.6 us with four waves).  Only where the
-    // resulting grid still fills the CUs evenly (37888 x 3584 would leave 296 workgroups on 256 CUs: 19.9 -> 22.8 us).
-    const int w8 = (strips + 7) / 8;
-    if (mt == 1 && M >= 8 && w8 >= 200 && ((w8 + 255) / 256) * 256 * 5 <= w8 * 6 && gemv_lookup(1, 8, 8) != nullptr) {
-        nt = 8;
-        nw = w8 > 256 ? 4 : 8;
-    }
     *nt_out = nt;
     *nw_out = nw;
 }
