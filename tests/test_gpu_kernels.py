@@ -181,6 +181,29 @@ def test_gemv_eight_column_tiles(ops, M, N, nw):
                          17, N, K, 128, cfg=(8, nw))
 
 
+@pytest.mark.parametrize("nt", [3, 5, 6, 7])
+@pytest.mark.parametrize("nw", [4, 8])
+def test_gemv_odd_column_tile_counts(ops, nt, nw):
+    """Column tiles per wave that do not divide the strip count: the last workgroup is ragged (33 strips)."""
+    N, K = 528, 1024
+    p = prep(N, K)
+    for M in (2, 16):
+        x = O.synth_acts(M, K, seed=M + nt)
+        out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128, cfg=(nt, nw))
+        assert O.max_abs_rel(host(out), O.gemm_f16(x, p["w16"])) < 2e-3
+
+
+@pytest.mark.parametrize("N", [4608, 10240, 28672])
+def test_gemv_default_split_on_unbalanced_widths(ops, N):
+    """Widths whose default is 2, 3 or 7 column tiles per wave; every M range of the default rule."""
+    K = 512
+    p = prep(N, K)
+    for M in (1, 8, 16, 32, 64):
+        x = O.synth_acts(M, K, seed=M)
+        out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+        assert O.max_abs_rel(host(out), O.gemm_f16(x, p["w16"])) < 2e-3
+
+
 def test_gemv_bias_and_ragged_strip(ops):
     N, K, M = 48, 256, 4                                    # N is not a multiple of the 64-column strip
     p = prep(N, K)
