@@ -180,9 +180,10 @@ int kmi_gemm_w8a8_tiled(void* out_f16, const void* a8, const void* w8_tiled, con
 int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, const void* bias,
                        int M, int N, int K, void* stream);
 
-/* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128 or 256. */
+/* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128, 256, or 192 (W8A8 and fp16 operand-copy
+ * lanes only: 256 rows x 128 columns, two workgroups per CU). */
 void kmi_gemm_force_tile(int tile);
-/* The workgroup tile (64, 128 or 256 rows) the automatic choice of the W8A8 lane uses for an M x N x K product.  With the 256 tile the library may run the columns of a
+/* The workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns) the automatic choice of the W8A8 lane uses for an M x N x K product.  With the 256 tile the library may run the columns of a
  * thin last round of tiles with the 128 tile in a second launch on the same stream (same results). */
 int kmi_gemm_pick_tile(int M, int N, int K);
 

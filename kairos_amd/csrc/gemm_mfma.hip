@@ -855,7 +855,8 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
 // already swizzled) makes the B side a straight 8 KiB copy per 128-row strip.
 
 template <int KIND, int BM, int BN, bool TILED_B, int NS>
-__global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((NS == 3 && BM == 256 && BN == 128) ? 2 : 1)))
+void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for two workgroups per CU: <= 256 registers, 72 KiB of LDS
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass cannot instantiate code that uses the buffer resource type
     constexpr bool I8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     static_assert(KIND == KIND_F16 || I8, "direct staging copies operands verbatim");
@@ -1062,14 +1063,14 @@ static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
     return s < 2 ? 1 : s;
 }
 
-template <int KIND, int BM, int BN, bool TILED>
+template <int KIND, int BM, int BN, bool TILED, int NS_ = 4>
 static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const bool whole = (a.n_begin == 0 && a.n_cols == a.N);
     constexpr bool DIRECT = (KIND == KIND_F16 || KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
-    constexpr int NS = 4;
+    constexpr int NS = NS_;
     constexpr size_t lds = DIRECT ? (size_t)NS * (BM + BN) * 64 : 2 * (size_t)(BM + BN) * 128;
     void (*fn)(GemmArgs);
     if constexpr (DIRECT) fn = gemm_direct_kernel<KIND, BM, BN, TILED, NS>;
@@ -1157,6 +1158,10 @@ static int pick_tile(int M, int N, long row_bytes) {
     if (split > row_bytes / 9000) split = row_bytes / 9000;
     if (split < 1) split = 1;
     if (M > 128 && wgs(256, 256) * split >= 144) return 256;
+    // too few 256 x 256 tiles for the CUs, yet the rows are too short to split: 256 x 128 tiles, two workgroups per CU
+    // (selector 192), when they come to 192..256 (2048 x 4096 x 14336: 119 against 130 us with 128 x 128 tiles and 134
+    // with 256 x 256; 1536 x 4096 x 14336: 95 against 106; on long rows the split 256 tile wins: 1024 x 8192 x 28672)
+    if (M >= 1024 && row_bytes <= 20000 && wgs(256, 256) < 144 && wgs(256, 128) >= 192 && wgs(256, 128) <= 256) return 192;
     const bool pad128 = (M + 127) / 128 * 2 > (M + 63) / 64;
     if (pad128 && wgs(64, 128) >= 200 && wgs(128, 128) < 256) return 64;
     if (M > 64 && wgs(128, 128) >= (row_bytes >= 8192 ? 48 : 144)) return 128;
@@ -1229,6 +1234,9 @@ static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
     }
     switch (tile) {
         case 256: return launch_gemm<KIND, 256, 256, TILED>(a, st);
+        case 192:                                        // 256 rows x 128 columns, three stages, two workgroups per CU
+            if constexpr (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16) return launch_gemm<KIND, 256, 128, TILED, 3>(a, st);
+            break;
         case 128: return launch_gemm<KIND, 128, 128, TILED>(a, st);
         case 64: return launch_gemm<KIND, 64, 128, TILED>(a, st);
     }

@@ -60,7 +60,8 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_gemm_w4a16_wp_rows(4096, 4096, 4096) == 0
     assert lib.kmi_gemm_pick_tile(4096, 4096, 4096) == 256 and lib.kmi_gemm_pick_tile(8, 4096, 4096) == 64
     assert lib.kmi_gemm_pick_tile(512, 4096, 4096) == 64 and lib.kmi_gemm_pick_tile(384, 4096, 14336) == 128
-    assert lib.kmi_gemm_pick_tile(768, 8192, 28672) == 256 and lib.kmi_gemm_pick_tile(2048, 4096, 14336) == 128   # split over K counts on long rows only
+    assert lib.kmi_gemm_pick_tile(768, 8192, 28672) == 256 and lib.kmi_gemm_pick_tile(1024, 4096, 14336) == 128   # split over K counts on long rows only
+    assert lib.kmi_gemm_pick_tile(2048, 4096, 14336) == 192 and lib.kmi_gemm_pick_tile(1024, 8192, 28672) == 256   # 256 x 128 tiles, two per CU
     assert lib.kmi_gemm_pick_tile(192, 10240, 8192) == 64 and lib.kmi_gemm_pick_tile(192, 28672, 4096) == 128      # row padding
     # offline weight preparation: same shape rules as the converters; table height is host arithmetic
     assert lib.kmi_prepare_weight(None, 8, 128, 128, 16, 16, 16, 16, 16, 16, None) == -1

@@ -289,7 +289,7 @@ def test_gemm_w4a16_f16_w8a16(ops, M, tile):
     assert O.max_abs_rel(host(out816), O.gemm_w8a16(x, p["w8"], p["scales_1"])) < 2e-3
 
 
-@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("tile", [64, 128, 192, 256])
 def test_gemm_tiled_operands_match_row_major(ops, tile):
     N, K, M = 384, 1024, 150
     p = prep(N, K)
@@ -669,7 +669,7 @@ def test_random_shapes_every_variant_agrees(ops):
         ws = torch.rand((N,), device="cuda", generator=g).to(torch.float16)
         outs = []
         try:
-            for tile in (0, 64, 128, 256):
+            for tile in (0, 64, 128, 192, 256):
                 ops.force_gemm_tile(tile)
                 o = torch.empty((M, N), device="cuda", dtype=torch.float16)
                 ops.w8a8_gemm_forward(a8, w8, ws, sx, o, bias=bias)
