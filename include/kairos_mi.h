@@ -202,6 +202,17 @@ int kmi_gemm_set_workspace(void* ptr, size_t bytes);
 /* Tuning hook for the calling thread: 0 = automatic split count, else the number of K splits. */
 void kmi_gemm_force_splits(int splits);
 
+/* ---- measurement aid ----------------------------------------------------------------------------- */
+
+/* No counterpart in the reference.  Runs `iters` rounds of sixteen independent v_mfma_i32_32x32x32_i8 (int8 != 0) or
+ * v_mfma_f32_32x32x16_f16 per wave, four waves per workgroup, entirely from registers, on operands read once from
+ * operands_32k (32 KiB: eight 16-byte values per thread of a workgroup).  sink_f32 needs workgroups*256 floats; clocks_2xi64 receives the shader clocks and the ticks
+ * of the constant 100 MHz counter that workgroup 0 spent in the loop (their ratio is the shader frequency).  Operations
+ * per launch: workgroups * 4 * iters * 16 * (int8 ? 65536 : 32768).  Used by `bench_extra mfmaceiling` to show what
+ * the matrix pipes sustain under the power limit with constant and with random operands. */
+int kmi_probe_mfma(int int8, const void* operands_32k, void* sink_f32, void* clocks_2xi64, int workgroups, int iters,
+                   void* stream);
+
 /* ---- interval lookup table (host only) --------------------------------------------------------- */
 
 /* Replaces LUT_module.LUT (kernels/csrc/kairos_kernel/lut/lut.h:8-45, lut_bindings.cpp:5-13).

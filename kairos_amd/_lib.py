@@ -42,6 +42,7 @@ SIGNATURES = {
     "kmi_gemm_w4a16_wp_rows": [_I, _I, _I],
     "kmi_gemm_set_workspace": [_P, ctypes.c_size_t],
     "kmi_gemm_force_splits": [_I],
+    "kmi_probe_mfma": [_I, _P, _P, _P, _I, _I, _P],
     "kmi_lut_new": [],
     "kmi_lut_free": [_P],
     "kmi_lut_record": [_P, _I, _I],

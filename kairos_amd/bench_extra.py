@@ -6,6 +6,7 @@
     python -m kairos_amd.bench_extra blasref   # the library's int8 / fp16 GEMMs of this image (hipBLASLt via torch) beside this build's
     python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
     python -m kairos_amd.bench_extra actnorm   # per-token quantiser and fused residual add + RMSNorm + quantiser, GB/s
+    python -m kairos_amd.bench_extra mfmaceiling  # register-only MFMA loops: the rate the GPU sustains under its power limit
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -258,6 +259,44 @@ def actnorm(args):
         torch.cuda.empty_cache()
     return {"bench": "actnorm", "rows": rows,
             "algorithmic_bytes": "2*M*K per fp16 tensor read or written, M*K + 2*M for the int8 form (gamma's 2*K not counted)"}
+
+
+def mfmaceiling(args):
+    """What the matrix pipes sustain on the whole GPU in a register-only loop (no memory traffic at all), with constant
+    and with random operands: the clock under full MFMA load is set by the power limit, and the power by the bits that
+    toggle.  The random-operand figure is the ceiling a GEMM of this library can reach on real data."""
+    dev = torch.device("cuda:0")
+    lib = ops._lib.load()
+    wgs, iters = 1024, 200000
+    sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
+    rows = []
+    for int8, name, ops_per_mfma, peak in ((1, "v_mfma_i32_32x32x32_i8", 65536, 5.0e15), (0, "v_mfma_f32_32x32x16_f16", 32768, 2.5e15)):
+        for data in ("constant", "random"):
+            if int8:                                       # 32 KiB of operands: eight 16-byte values per thread
+                src = (torch.full((8192,), 0x01010101, dtype=torch.int32) if data == "constant"
+                       else torch.randint(-2 ** 31, 2 ** 31 - 1, (8192,), dtype=torch.int32))
+            else:
+                h = (torch.ones(16384, dtype=torch.float16) if data == "constant"
+                     else (torch.rand(16384) * 0.5 + 0.125).to(torch.float16) * (torch.randint(0, 2, (16384,)) * 2 - 1).to(torch.float16))
+                src = h.view(torch.int32)
+            assert src.numel() * 4 == 32768
+            src = src.to(dev)
+            best = None
+            for _ in range(3):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                ops._lib.check(lib.kmi_probe_mfma(int8, src.data_ptr(), sink.data_ptr(), clk.data_ptr(), wgs, iters, ops._stream()))
+                b.record()
+                torch.cuda.synchronize()
+                sec = a.elapsed_time(b) * 1e-3
+                best = sec if best is None or sec < best else best
+            c = clk.cpu()
+            rate = wgs * 4 * iters * 16 * ops_per_mfma / best
+            rows.append({"instruction": name, "operands": data, "ms": round(best * 1e3, 2), "tops": round(rate / 1e12, 1),
+                         "frac_of_published_peak": round(rate / peak, 4), "shader_mhz": round(float(c[0]) / float(c[1]) * 100.0, 0)})
+            print(rows[-1], file=sys.stderr, flush=True)
+    return {"bench": "mfmaceiling", "workgroups": wgs, "waves_per_workgroup": 4, "iters": iters, "rows": rows}
 
 
 # ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
@@ -534,6 +573,7 @@ def main(argv=None):
     sub.add_parser("weightprep")
     sub.add_parser("blasref")
     sub.add_parser("actnorm")
+    sub.add_parser("mfmaceiling")
     d = sub.add_parser("decoder")
     d.add_argument("--lut", default=None)
     d.add_argument("--layers", type=int, default=32)
@@ -551,7 +591,7 @@ def main(argv=None):
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
     ops.ensure_workspace()
-    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "mfmaceiling": mfmaceiling, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

@@ -90,6 +90,7 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_silu_mul_quant_act(None, None, 8, 16, 2, 128, None) == -5
     assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 2, 100, None) == -2
     assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 0, 128, None) == 0
+    assert lib.kmi_probe_mfma(1, None, 16, 16, 4, 4, None) == -1 and lib.kmi_probe_mfma(1, 16, 16, 16, 0, 4, None) == -2
     assert lib.kmi_lut_get(None, 3) == -7
 
 
