@@ -296,7 +296,27 @@ def mfmaceiling(args):
             rows.append({"instruction": name, "operands": data, "ms": round(best * 1e3, 2), "tops": round(rate / 1e12, 1),
                          "frac_of_published_peak": round(rate / peak, 4), "shader_mhz": round(float(c[0]) / float(c[1]) * 100.0, 0)})
             print(rows[-1], file=sys.stderr, flush=True)
-    return {"bench": "mfmaceiling", "workgroups": wgs, "waves_per_workgroup": 4, "iters": iters, "rows": rows}
+    # the dominant GEMM itself (W8A8, 256 x 256 tile, row-major weights) on operands of different bit activity: same
+    # kernel, same schedule, the difference is the clock the power limit allows
+    M, N, K = 4096, 28672, 4096
+    ws = torch.rand(N, device=dev, dtype=torch.float16)
+    asc = torch.rand(M, device=dev, dtype=torch.float16)
+    out = torch.empty((M, N), device=dev, dtype=torch.float16)
+
+    def operand(kind, shape):
+        if kind == "zeros":
+            return torch.zeros(shape, dtype=torch.int8, device=dev)
+        lo, hi = (-3, 4) if kind == "small (-3..3)" else (-128, 128)
+        return torch.randint(lo, hi, shape, dtype=torch.int8, device=dev)
+    gemm_rows = []
+    for ak, wk in (("zeros", "zeros"), ("zeros", "random"), ("small (-3..3)", "small (-3..3)"), ("small (-3..3)", "random"), ("random", "random")):
+        a8 = [operand(ak, (M, K)) for _ in range(2)]
+        w8 = [operand(wk, (N, K)) for _ in range(2)]
+        us = _time(lambda i: ops.w8a8_gemm_forward(a8[i & 1], w8[i & 1], ws, asc, out), 30)
+        gemm_rows.append({"M": M, "N": N, "K": K, "activations": ak, "weights": wk, "us": round(us, 1),
+                          "tops": round(2.0 * M * N * K / us / 1e6, 1), "frac_of_published_peak": round(2.0 * M * N * K / us / 1e-6 / 5.0e15, 4)})
+        print(gemm_rows[-1], file=sys.stderr, flush=True)
+    return {"bench": "mfmaceiling", "workgroups": wgs, "waves_per_workgroup": 4, "iters": iters, "rows": rows, "gemm_rows": gemm_rows}
 
 
 # ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
