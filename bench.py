@@ -26,10 +26,25 @@ LAYER = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), 
 M_GRID = [1 << i for i in range(13)]
 PEAK = {"hbm": 8.0e12, "f16": 2.5e15, "i8": 5.0e15}       # MI355X published: HBM3E B/s, dense MFMA op/s
 LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x")
-# HBM<->L2 bytes per launch of the dominant kernel, from the committed counter runs (profiles/
-# bench_llama3_8b_fetch_write_size.md): mean over the calls of one step (tail launches included), 2.0*FETCH_SIZE + WRITE_SIZE KiB.
-MEASURED_TRAFFIC = {"gemm_w8a8[256]": int((2.0 * 137787 + 71171) * 1024)}
+# HBM<->L2 bytes per call of the dominant kernel: written by `python -m kairos_amd.traffic` from two rocprofv3 counter
+# runs of this script (--only-label), stamped with a hash of the kernel sources; ignored once the sources change.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_llama3_8b_traffic.json")
 G = 128
+
+
+def synth_weights(torch, N, K, seed=10):
+    """fp16 N(0, 0.02) [N, K], seeded on the host so that every box sees the same weights."""
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn((N, K), generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+
+
+def synth_acts(torch, M, K, seed=11):
+    """fp16 N(0, 1) [M, K] with a fixed 1 % of the K channels scaled x20 (outliers)."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((M, K), generator=g, dtype=torch.float32)
+    cols = torch.randperm(K, generator=g)[: int(0.01 * K)]
+    x[:, cols] *= 20.0
+    return x.to(torch.float16)
 
 
 def algorithmic(kernel, M, N, K):
@@ -119,45 +134,67 @@ class Tracer:
         return agg
 
 
-def cpu_baseline(gpu_us_per_layer_m16):
-    """The oracle's W4A16 lane (dequantise, then fp32-accumulated matmul) for the four linears of the layer at
-    M = 16, one thread: the same unit as `value`, directly comparable with the M = 16 entry of the per-M table."""
+def cpu_baseline(gpu_us_per_layer_by_m):
+    """The oracle's W4A16 lane (unpack, fp16 FMA dequantisation, fp32-accumulated matmul) for the four linears of the
+    layer, on the host cores of this box: the same unit as `value`, comparable with the per-M table.  The oracle's own
+    functions run on column slabs of the weight, one slab per worker thread (numpy releases the interpreter lock
+    inside its loops); BLAS is held to one thread per worker.  Also timed on a single thread."""
     import numpy as np
+    from concurrent.futures import ThreadPoolExecutor
     from oracle import kairos_oracle as O
     try:
         from threadpoolctl import threadpool_limits
     except ImportError:                                      # pragma: no cover
         threadpool_limits = None
-    M = 16
+    cores = os.cpu_count() or 1
+    for var in ("OMP_NUM_THREADS", "MAX_JOBS"):              # the box's CPU share, when it says so
+        if os.environ.get(var, "").isdigit():
+            cores = min(cores, int(os.environ[var]))
     rng = np.random.default_rng(10)
-    work = []
+    weights = []
     for _name, N, K in LAYER:                                # random packed weights: the timing does not depend on the values
         gp = O.padded_groups(K)
         qw = rng.integers(-32768, 32768, size=(N // 4, K), dtype=np.int16)
         sc = (rng.random((gp, N), dtype=np.float32) * 0.01 + 0.002).astype(np.float16)
         sz = (-(sc.astype(np.float32) * 7.5)).astype(np.float16)
-        work.append((O.synth_acts(M, K), qw, sc, sz))
+        weights.append((N, K, qw, sc, sz))
+    acts = {(M, K): O.synth_acts(M, K) for M in (16, 1024) for K in sorted({k for _, _, k in LAYER})}
+    SLAB = 256                                               # weight rows per task (a multiple of the 4-row interleave)
 
-    def once():
+    def layer(M, pool):
         t0 = time.perf_counter()
-        for x, qw, sc, sz in work:
-            O.gemm_w4a16(x, qw, sc, sz)
+        for N, K, qw, sc, sz in weights:
+            x = acts[(M, K)]
+            job = lambda r0: O.gemm_w4a16(x, qw[r0 // 4:(r0 + SLAB) // 4], sc[:, r0:r0 + SLAB], sz[:, r0:r0 + SLAB])
+            starts = range(0, N, SLAB)
+            parts = list(pool.map(job, starts)) if pool else [job(r) for r in starts]
+            assert sum(p.shape[1] for p in parts) == N
         return time.perf_counter() - t0
+
+    def median_of(M, pool, passes):
+        layer(M, pool)
+        ts = sorted(layer(M, pool) for _ in range(passes))
+        return ts[len(ts) // 2], sum(ts)
 
     ctx = threadpool_limits(limits=1) if threadpool_limits else None
     if ctx:
         ctx.__enter__()
     try:
-        once()
-        ts = sorted(once() for _ in range(9))
+        with ThreadPoolExecutor(max_workers=cores) as pool:
+            m16, w16 = median_of(16, pool, 7)
+            m1k, w1k = median_of(1024, pool, 3)
+        one, w1 = median_of(16, None, 3)
     finally:
         if ctx:
             ctx.__exit__(None, None, None)
-    med = ts[len(ts) // 2]
-    return {"value": med * 1e6, "unit": "us/layer at M=16 (W4A16 lane)", "cores": 1, "kind": "port",
-            "sample": f"numpy oracle, dequantise + matmul of the layer's four linears at M=16, one thread, ten passes "
-                      f"({sum(ts) + med:.1f} s of CPU work, median {med * 1e3:.0f} ms per layer); the GPU spends "
-                      f"{gpu_us_per_layer_m16:.1f} us on the same layer at M=16"}
+    return {"value": m16 * 1e6, "unit": "us/layer at M=16 (W4A16 lane)", "cores": cores, "kind": "port",
+            "by_m_us_per_layer": {"16": round(m16 * 1e6), "1024": round(m1k * 1e6)},
+            "one_thread_us_per_layer_m16": round(one * 1e6),
+            "sample": f"numpy oracle (unpack, fp16-FMA dequantise, fp32 matmul) of the layer's four linears on {cores} "
+                      f"worker threads over {SLAB}-row weight slabs: M=16 median of 7 passes {m16 * 1e3:.0f} ms, M=1024 "
+                      f"median of 3 passes {m1k * 1e3:.0f} ms; one thread at M=16 {one * 1e3:.0f} ms "
+                      f"(about {w16 + w1k + w1 + m16 + m1k + one:.0f} s of wall time in all); the GPU spends "
+                      f"{gpu_us_per_layer_by_m[16]:.1f} us at M=16 and {gpu_us_per_layer_by_m[1024]:.1f} us at M=1024 on the same layer"}
 
 
 def main():
@@ -177,6 +214,10 @@ def main():
     ap.add_argument("--out", default=None, help="where to write the per-lane sweep table (JSON)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--only-label", default=None,
+                    help="counter runs: after set-up, run only the calls of the step that are booked under this kernel "
+                         "label (e.g. 'gemm_w8a8[256]'), --steps times, and exit without the JSON line")
+    ap.add_argument("--calls-json", default=None, help="with --only-label: where to write the number of calls made")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on one GPU (every linear is independent and would shard by columns "
@@ -190,7 +231,7 @@ def main():
     from kairos_amd import ops
     from kairos_amd.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
     from kairos_amd.perf_profiler import Profiler
-    from oracle import kairos_oracle as O                     # synthetic inputs + the CPU leg only
+    from kairos_amd import traffic
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -203,7 +244,7 @@ def main():
     # ---- synthetic layer copies --------------------------------------------------------------
     layers = []
     for _name, N, K in LAYER:
-        prep = ops.prepare_weight(torch.from_numpy(O.synth_weights(N, K, seed=10)).to(dev))
+        prep = ops.prepare_weight(synth_weights(torch, N, K, seed=10).to(dev))
         copies = []
         for c in range(args.copies):
             dl = DynamicLinear(K, N, False, dev, 128)
@@ -214,7 +255,7 @@ def main():
     acts = {}
     for K in sorted({k for _, _, k in LAYER}):
         for M in M_GRID:
-            acts[(M, K)] = torch.from_numpy(O.synth_acts(M, K, seed=11)).to(dev).reshape(1, M, K)
+            acts[(M, K)] = synth_acts(torch, M, K, seed=11).to(dev).reshape(1, M, K)
 
     if args.calib_copy:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
@@ -244,6 +285,31 @@ def main():
             c = (s * len(M_GRID) + mi) % args.copies
             for li, (_n, _N, K) in enumerate(LAYER):
                 layers[li][c](acts[(M, K)])
+
+    # ---- counter runs: only the calls booked under one kernel label -----------------------------
+    if args.only_label:
+        picks = []
+        for M in M_GRID:
+            for li, (_n, N, K) in enumerate(LAYER):
+                lane = names[prof.get_comp_type((N, K), M)]
+                kern = {"w4a16_gemv": "gemv_w4a16", "w4a16_gemm": "gemm_w4a16", "w8a8": "gemm_w8a8",
+                        "w8a16_gemm": "gemm_w8a16", "fp16": "gemm_f16"}[lane]
+                probe = Tracer(torch, ops)
+                probe.begin(kern, M, N, K)
+                if probe._cur[0] == args.only_label:
+                    picks.append((M, li, K, algorithmic(kern, M, N, K)[0]))
+        if not picks:
+            sys.exit(f"bench.py: no call of the step is booked under {args.only_label}")
+        for s in range(args.warmup + args.steps):
+            for M, li, K, _b in picks:
+                layers[li][s % args.copies](acts[(M, K)])
+        torch.cuda.synchronize()
+        if args.calls_json:
+            with open(args.calls_json, "w") as f:
+                json.dump({"label": args.only_label, "calls": len(picks) * (args.warmup + args.steps),
+                           "algorithmic_bytes_per_call": int(sum(b for *_r, b in picks) / len(picks)),
+                           "shapes": [[M, LAYER[li][1], K] for M, li, K, _b in picks]}, f)
+        return
 
     # ---- timed region -------------------------------------------------------------------------
     for s in range(args.warmup):
@@ -288,8 +354,10 @@ def main():
         achieved, peak, unit, bound = dom["flops"] / dom["sec"] / 1e12, PEAK[dom["dt"]] / 1e12, "TFLOP/s", "mfma"
     else:
         achieved, peak, unit, bound = dom["bytes"] / dom["sec"] / 1e9, PEAK["hbm"] / 1e9, "GB/s", "hbm"
+    traffic_bytes, traffic_note = traffic.load(dom_label, TRAFFIC_FILE)
     roofline = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(dom_label), "kernel": dom_label,
+                "frac": round(achieved / peak, 4), "traffic": traffic_bytes, "traffic_source": traffic_note,
+                "kernel": dom_label,
                 "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
                 "launches": dom["launches"], "avg_launch_us": round(avg_dur * 1e6, 2),
                 "share_of_kernel_time": round(dom["sec"] / total_kernel_sec, 4)}
@@ -384,7 +452,7 @@ def main():
 
     # the GPU on the CPU leg's sample: config 1 through the small-M lane
     cfg1_us = time_calls(lambda i=0: layers[1][i % args.copies]._forward(acts[(16, 4096)], 16, COMP_TYPE_NAME["w4a16_gemv"]), 50)
-    cpu = None if args.no_cpu else cpu_baseline(by_m[16])
+    cpu = None if args.no_cpu else cpu_baseline(by_m)
 
     result = {
         "metric": "switched mpGEMM us/layer over M=1..4096, Llama-3-8B shapes",

@@ -2,8 +2,11 @@
  * kairos_mi.h -- C ABI of the MI355X (gfx950) switched mixed-precision linear path.
  *
  * Every entry point takes raw DEVICE pointers, sizes and a HIP stream (passed as void*, i.e. a
- * hipStream_t; NULL = the null stream).  The caller owns and allocates every buffer, outputs
- * included; nothing here allocates, frees or synchronises.  All functions are re-entrant.
+ * hipStream_t; NULL = the null stream).  The caller owns and allocates every buffer, outputs and
+ * scratch included; nothing here allocates, frees or synchronises, and no call leaves state behind
+ * that a later call's result depends on.  Functions may be called from any host thread; the only
+ * per-thread state is the last error message and the test hooks kmi_gemm_force_tile /
+ * kmi_gemm_force_splits (marked below).  A LUT handle must not be used from two threads at once.
  * Return value: KMI_OK (0) or a negative KMI_E_* code; kmi_get_last_error_string() gives the
  * calling thread's last message.  Nothing throws across this boundary.
  *
@@ -148,70 +151,70 @@ int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, co
                        const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
                        int nt, int nw, void* stream);
 
-/* ---- MFMA GEMMs, any M ------------------------------------------------------------------------- */
+/* ---- MFMA GEMMs, any M -------------------------------------------------------------------------
+ *
+ * Every GEMM entry point ends with (workspace, workspace_bytes, stream).  workspace is optional caller-owned device
+ * scratch (16-byte aligned; NULL = none) for split-K: when the output tiles alone cannot fill the GPU (mid-sized M)
+ * the call writes fp32 / int32 partial sums there and reduces them with a second kernel on the same stream, in a
+ * fixed order (deterministic).  The library keeps no reference to it after the call's launches; calls that share
+ * one buffer must be ordered on one stream.  The number of splits depends on the arguments only (shape, buffer
+ * size; kmi_gemm_splits_for reports it), never on earlier calls or on the calling thread; the int8 lane's results
+ * do not depend on it at all, the fp16 lanes' fp32 summation order does.  64 MiB covers every split the library
+ * would choose for outputs up to 2 Mi elements. */
 
 /* W4A16: replaces gemm_forward_cuda_new (thirdparty/AWQ/kernels/csrc/pybind.cpp:22,
  * thirdparty/AWQ/kernels/csrc/quantization_new/gemm/gemm_cuda.cu:1126-1235); the caller supplies out. */
 int kmi_gemm_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
-                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
+                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
 /* W8A16: out = fp16((x . w8^T) * wscales[n]) (+bias).  The reference only declares the ids
  * (kairos/dynamic_linear.py:8-9). */
 int kmi_gemm_w8a16(void* out_f16, const void* x_f16, const void* w8, const void* wscales_f16,
-                   const void* bias, int M, int N, int K, void* stream);
+                   const void* bias, int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 
 /* W8A8: acc = a8 . w8^T in int32; out = fp16(float(acc) * (float(wscales[n]) * float(ascales[m]))) (+bias).
  * Replaces w8a8_gemm_forward_cuda (thirdparty/AWQ/kernels/csrc/pybind.cpp:21,
  * thirdparty/AWQ/kernels/csrc/w8a8/w8a8_gemm_cuda.cu:909-954). */
 int kmi_gemm_w8a8(void* out_f16, const void* a8, const void* w8, const void* wscales_f16,
-                  const void* ascales_f16, const void* bias, int M, int N, int K, void* stream);
+                  const void* ascales_f16, const void* bias, int M, int N, int K,
+                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* The same product with the raw int32 accumulators written out [M, N] (bit-exact tier). */
-int kmi_gemm_w8a8_acc_i32(void* acc_i32, const void* a8, const void* w8, int M, int N, int K, void* stream);
+int kmi_gemm_w8a8_acc_i32(void* acc_i32, const void* a8, const void* w8, int M, int N, int K,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* FP16: out = x . w16^T (+bias), fp32 accumulation.  Replaces `input @ tmp_weight.T`
  * (kairos/dynamic_linear.py:163). */
 int kmi_gemm_f16(void* out_f16, const void* x_f16, const void* w16, const void* bias,
-                 int M, int N, int K, void* stream);
+                 int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Variants reading the weight operand in the tiled layout written by kmi_cvt_*_tiled. */
 int kmi_gemm_w8a8_tiled(void* out_f16, const void* a8, const void* w8_tiled, const void* wscales_f16,
-                        const void* ascales_f16, const void* bias, int M, int N, int K, void* stream);
+                        const void* ascales_f16, const void* bias, int M, int N, int K,
+                        void* workspace, size_t workspace_bytes, void* stream);
 int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, const void* bias,
-                       int M, int N, int K, void* stream);
+                       int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Tuning hook for the calling thread: 0 = automatic tile choice, else 64, 128, 256, or 192 (W8A8 and fp16 operand-copy
- * lanes only: 256 rows x 128 columns, two workgroups per CU). */
-void kmi_gemm_force_tile(int tile);
-/* The workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns) the automatic choice of the W8A8 lane uses for an M x N x K product.  With the 256 tile the library may run the columns of a
- * thin last round of tiles with the 128 tile in a second launch on the same stream (same results). */
+/* Host-only queries of the automatic choices (no GPU work).
+ * kmi_gemm_pick_tile: the workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns) of the W8A8 lane for an
+ *   M x N x K product.  With the 256 tile the library may run the columns of a thin last round of tiles with the 128
+ *   tile in a second launch on the same stream (same results).
+ * kmi_gemm_w4a16_wp_rows: rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses (weights decoded in
+ *   registers by the wave that owns their columns), or 0 when the LDS-staged variant runs.
+ * kmi_gemm_splits_for: K splits a call would use with a workspace of that many bytes (1 = none); lane 0 = W4A16,
+ *   1 = W8A16, 2 = W8A8, 3 = fp16. */
 int kmi_gemm_pick_tile(int M, int N, int K);
-
-/* Rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses for an M x N x K product (weights decoded
- * in registers by the wave that owns their columns), or 0 when the LDS-staged variant runs.  Forcing: tile
- * selectors 1032 / 1064 / 1128 (two wave quartets per workgroup) and 2032 / 2064 / 2128 (one) in
- * kmi_gemm_force_tile. */
 int kmi_gemm_w4a16_wp_rows(int M, int N, int K);
+int kmi_gemm_splits_for(int lane, int M, int N, int K, size_t workspace_bytes);
 
-/* Optional scratch for split-K (used when the output tiles alone cannot fill the GPU, i.e. mid-sized
- * M): the calling thread registers a caller-owned device buffer; GEMM calls made by that thread then
- * write fp32/int32 partial sums there and reduce them with a second kernel on the same stream, in a
- * fixed order (deterministic).  The buffer must outlive those calls; calls that share it must be
- * ordered on one stream.  ptr = NULL unregisters.  No reference counterpart. */
-int kmi_gemm_set_workspace(void* ptr, size_t bytes);
-/* Tuning hook for the calling thread: 0 = automatic split count, else the number of K splits. */
+/* TEST AND TUNING HOOKS (state of the calling host thread, 0 = automatic; production callers never set them).
+ * kmi_gemm_force_tile: 64, 128, 256, or 192 (W8A8 and fp16 operand-copy lanes only: 256 rows x 128 columns, two
+ *   workgroups per CU); for kmi_gemm_w4a16 also 1032 / 1064 / 1128 (small-M variant, two wave quartets per
+ *   workgroup) and 2032 / 2064 / 2128 (one).
+ * kmi_gemm_force_splits: the number of K splits (needs a workspace in the call). */
+void kmi_gemm_force_tile(int tile);
 void kmi_gemm_force_splits(int splits);
-
-/* ---- measurement aid ----------------------------------------------------------------------------- */
-
-/* No counterpart in the reference.  Runs `iters` rounds of sixteen independent v_mfma_i32_32x32x32_i8 (int8 != 0) or
- * v_mfma_f32_32x32x16_f16 per wave, four waves per workgroup, entirely from registers, on operands read once from
- * operands_32k (32 KiB: eight 16-byte values per thread of a workgroup).  sink_f32 needs workgroups*256 floats; clocks_2xi64 receives the shader clocks and the ticks
- * of the constant 100 MHz counter that workgroup 0 spent in the loop (their ratio is the shader frequency).  Operations
- * per launch: workgroups * 4 * iters * 16 * (int8 ? 65536 : 32768).  Used by `bench_extra mfmaceiling` to show what
- * the matrix pipes sustain under the power limit with constant and with random operands. */
-int kmi_probe_mfma(int int8, const void* operands_32k, void* sink_f32, void* clocks_2xi64, int workgroups, int iters,
-                   void* stream);
 
 /* ---- interval lookup table (host only) --------------------------------------------------------- */
 

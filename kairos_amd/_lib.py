@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libkairos_mi.so")
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
+_Z = ctypes.c_size_t
 
 # name -> argument types (every function returns int unless listed in _RESTYPE)
 SIGNATURES = {
@@ -30,19 +31,19 @@ SIGNATURES = {
     "kmi_trans_layout_w4a8": [_P, _P, _I, _I, _P],
     "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-    "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "kmi_gemm_w8a16": [_P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_w8a8": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_w8a8_acc_i32": [_P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_f16": [_P, _P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P],
+    # GEMMs end with (workspace pointer, workspace bytes, stream)
+    "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w8a16": [_P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w8a8": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w8a8_acc_i32": [_P, _P, _P, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_f16": [_P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_force_tile": [_I],
     "kmi_gemm_pick_tile": [_I, _I, _I],
     "kmi_gemm_w4a16_wp_rows": [_I, _I, _I],
-    "kmi_gemm_set_workspace": [_P, ctypes.c_size_t],
+    "kmi_gemm_splits_for": [_I, _I, _I, _I, _Z],
     "kmi_gemm_force_splits": [_I],
-    "kmi_probe_mfma": [_I, _P, _P, _P, _I, _I, _P],
     "kmi_lut_new": [],
     "kmi_lut_free": [_P],
     "kmi_lut_record": [_P, _I, _I],

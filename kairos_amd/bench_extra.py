@@ -6,7 +6,6 @@
     python -m kairos_amd.bench_extra blasref   # the library's int8 / fp16 GEMMs of this image (hipBLASLt via torch) beside this build's
     python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
     python -m kairos_amd.bench_extra actnorm   # per-token quantiser and fused residual add + RMSNorm + quantiser, GB/s
-    python -m kairos_amd.bench_extra mfmaceiling  # register-only MFMA loops: the rate the GPU sustains under its power limit
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -261,64 +260,6 @@ def actnorm(args):
             "algorithmic_bytes": "2*M*K per fp16 tensor read or written, M*K + 2*M for the int8 form (gamma's 2*K not counted)"}
 
 
-def mfmaceiling(args):
-    """What the matrix pipes sustain on the whole GPU in a register-only loop (no memory traffic at all), with constant
-    and with random operands: the clock under full MFMA load is set by the power limit, and the power by the bits that
-    toggle.  The random-operand figure is the ceiling a GEMM of this library can reach on real data."""
-    dev = torch.device("cuda:0")
-    lib = ops._lib.load()
-    wgs, iters = 1024, 200000
-    sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
-    clk = torch.zeros(2, dtype=torch.int64, device=dev)
-    rows = []
-    for int8, name, ops_per_mfma, peak in ((1, "v_mfma_i32_32x32x32_i8", 65536, 5.0e15), (0, "v_mfma_f32_32x32x16_f16", 32768, 2.5e15)):
-        for data in ("constant", "random"):
-            if int8:                                       # 32 KiB of operands: eight 16-byte values per thread
-                src = (torch.full((8192,), 0x01010101, dtype=torch.int32) if data == "constant"
-                       else torch.randint(-2 ** 31, 2 ** 31 - 1, (8192,), dtype=torch.int32))
-            else:
-                h = (torch.ones(16384, dtype=torch.float16) if data == "constant"
-                     else (torch.rand(16384) * 0.5 + 0.125).to(torch.float16) * (torch.randint(0, 2, (16384,)) * 2 - 1).to(torch.float16))
-                src = h.view(torch.int32)
-            assert src.numel() * 4 == 32768
-            src = src.to(dev)
-            best = None
-            for _ in range(3):
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                ops._lib.check(lib.kmi_probe_mfma(int8, src.data_ptr(), sink.data_ptr(), clk.data_ptr(), wgs, iters, ops._stream()))
-                b.record()
-                torch.cuda.synchronize()
-                sec = a.elapsed_time(b) * 1e-3
-                best = sec if best is None or sec < best else best
-            c = clk.cpu()
-            rate = wgs * 4 * iters * 16 * ops_per_mfma / best
-            rows.append({"instruction": name, "operands": data, "ms": round(best * 1e3, 2), "tops": round(rate / 1e12, 1),
-                         "frac_of_published_peak": round(rate / peak, 4), "shader_mhz": round(float(c[0]) / float(c[1]) * 100.0, 0)})
-            print(rows[-1], file=sys.stderr, flush=True)
-    # the dominant GEMM itself (W8A8, 256 x 256 tile, row-major weights) on operands of different bit activity: same
-    # kernel, same schedule, the difference is the clock the power limit allows
-    M, N, K = 4096, 28672, 4096
-    ws = torch.rand(N, device=dev, dtype=torch.float16)
-    asc = torch.rand(M, device=dev, dtype=torch.float16)
-    out = torch.empty((M, N), device=dev, dtype=torch.float16)
-
-    def operand(kind, shape):
-        if kind == "zeros":
-            return torch.zeros(shape, dtype=torch.int8, device=dev)
-        lo, hi = (-3, 4) if kind == "small (-3..3)" else (-128, 128)
-        return torch.randint(lo, hi, shape, dtype=torch.int8, device=dev)
-    gemm_rows = []
-    for ak, wk in (("zeros", "zeros"), ("zeros", "random"), ("small (-3..3)", "small (-3..3)"), ("small (-3..3)", "random"), ("random", "random")):
-        a8 = [operand(ak, (M, K)) for _ in range(2)]
-        w8 = [operand(wk, (N, K)) for _ in range(2)]
-        us = _time(lambda i: ops.w8a8_gemm_forward(a8[i & 1], w8[i & 1], ws, asc, out), 30)
-        gemm_rows.append({"M": M, "N": N, "K": K, "activations": ak, "weights": wk, "us": round(us, 1),
-                          "tops": round(2.0 * M * N * K / us / 1e6, 1), "frac_of_published_peak": round(2.0 * M * N * K / us / 1e-6 / 5.0e15, 4)})
-        print(gemm_rows[-1], file=sys.stderr, flush=True)
-    return {"bench": "mfmaceiling", "workgroups": wgs, "waves_per_workgroup": 4, "iters": iters, "rows": rows, "gemm_rows": gemm_rows}
-
-
 # ---- config 5: random-init Llama-3-8B decoder -------------------------------------------------------
 class _RMSNorm(torch.nn.Module):
     def __init__(self, dim, dev):
@@ -446,6 +387,79 @@ class _Layer(torch.nn.Module):
         return self._mlp(x, a.view(B, self.h, 1, self.d))
 
 
+class Decoder:
+    """Random-init decoder stack over switched linears: embedding, `layers` x _Layer, final norm, vocabulary
+    projection, greedy pick.  `linears[l]` = (qkv, o, gate_up, down) callables of layer l.  The decode step has fixed
+    shapes (static KV cache, device-side position), so `capture()` records it into one HIP graph."""
+
+    def __init__(self, linears, dev, hidden=4096, heads=32, kv_heads=8, vocab=128256, matched=True, t_max=2048, seed=0):
+        self.dev, self.hidden, self.vocab, self.t_max = dev, hidden, vocab, t_max
+        self.head_dim = hidden // heads
+        self.layers = [_Layer(lin, dev, hidden, heads, kv_heads, matched=matched) for lin in linears]
+        g = torch.Generator(device=dev).manual_seed(seed)
+        self.emb = torch.randn(vocab, hidden, generator=g, device=dev, dtype=torch.float16) * 0.02
+        self.head = torch.randn(vocab, hidden, generator=g, device=dev, dtype=torch.float16) * 0.02
+        self.fnorm = _RMSNorm(hidden, dev)
+        self.ar = torch.arange(t_max, device=dev)
+        self.graph = None
+
+    def alloc(self, B):
+        for L in self.layers:
+            L.alloc_cache(B, self.t_max, self.dev)
+        self.x_in = torch.zeros((B, 1, self.hidden), dtype=torch.float16, device=self.dev)   # static buffers of the step
+        self.pos = torch.zeros((1,), dtype=torch.int64, device=self.dev)
+        self.tok = torch.zeros((B, 1), dtype=torch.int64, device=self.dev)
+        self.logits = torch.zeros((B, 1, self.vocab), dtype=torch.float16, device=self.dev)
+        self.graph = None
+
+    def free(self):
+        self.graph = None
+        for L in self.layers:
+            L.k_cache = L.v_cache = None
+        torch.cuda.empty_cache()
+
+    @torch.no_grad()
+    def prefill_logits(self, ids):
+        h, delta = self.emb[ids], None
+        for L in self.layers:
+            h, delta = L.prefill(h, delta)
+        return self.fnorm(h[:, -1:, :] + delta[:, -1:, :]) @ self.head.T                     # [B, 1, vocab]
+
+    def prefill(self, ids):
+        return self.prefill_logits(ids).argmax(-1)                                           # [B, 1]
+
+    @torch.no_grad()
+    def step(self):
+        mask = (self.ar <= self.pos).view(1, 1, 1, self.t_max)
+        cs = _rope_table(self.pos, self.head_dim, self.dev)
+        h, delta = self.x_in, None
+        for L in self.layers:
+            h, delta = L.step(h, delta, self.pos, mask, cs)
+        self.logits.copy_(self.fnorm(h + delta) @ self.head.T)
+        nxt = self.logits.argmax(-1)
+        self.tok.copy_(nxt)
+        self.x_in.copy_(self.emb[nxt])
+        self.pos.add_(1)
+
+    def start(self, first, prompt_len):
+        self.x_in.copy_(self.emb[first])
+        self.pos.fill_(prompt_len)
+
+    def capture(self):
+        """One warm-up step on a side stream, then the step recorded on that stream (its split-K scratch and the
+        temp cache exist by then).  The caller re-starts the sequence afterwards."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            self.step()
+        return self.graph
+
+
 def decoder(args):
     """End-to-end decoder: 32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336, vocab 128256; every linear a
     LUT-switched DynamicLinear (fused qkv and gate_up); protocol of utils/perf_eval.py:235-275.  The decode step
@@ -459,74 +473,34 @@ def decoder(args):
     DynamicLinear.prof = prof
     nl = args.layers
     per_shape = [_layer(N, K, nl, dev) for N, K in shapes]
-    layers = [_Layer([per_shape[s][l] for s in range(4)], dev, matched=not args.torch_norm) for l in range(nl)]
-    vocab = 128256
-    emb = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
-    head = (torch.randn(vocab, 4096, device=dev, dtype=torch.float16) * 0.02)
-    fnorm = _RMSNorm(4096, dev)
-    t_max = args.prompt + args.new_tokens + 8
-    ar = torch.arange(t_max, device=dev)
+    dec = Decoder([[per_shape[s][l] for s in range(4)] for l in range(nl)], dev, matched=not args.torch_norm,
+                  t_max=args.prompt + args.new_tokens + 8)
+    layers, vocab = dec.layers, dec.vocab
     names = {v: k for k, v in COMP_TYPE_NAME.items()}
-
-    @torch.no_grad()
-    def prefill(ids):
-        h, delta = emb[ids], None
-        for L in layers:
-            h, delta = L.prefill(h, delta)
-        return (fnorm(h[:, -1:, :] + delta[:, -1:, :]) @ head.T).argmax(-1)    # [B, 1]
 
     results = []
     for B in args.batches:
-        for L in layers:
-            L.alloc_cache(B, t_max, dev)
+        dec.alloc(B)
         ids = torch.randint(0, vocab, (B, args.prompt), device=dev)
-        x_in = torch.zeros((B, 1, 4096), dtype=torch.float16, device=dev)   # static buffers of the step
-        pos = torch.zeros((1,), dtype=torch.int64, device=dev)
-        tok = torch.zeros((B, 1), dtype=torch.int64, device=dev)
-
-        @torch.no_grad()
-        def step():
-            mask = (ar <= pos).view(1, 1, 1, t_max)
-            cs = _rope_table(pos, 128, dev)
-            h, delta = x_in, None
-            for L in layers:
-                h, delta = L.step(h, delta, pos, mask, cs)
-            nxt = (fnorm(h + delta) @ head.T).argmax(-1)
-            tok.copy_(nxt)
-            x_in.copy_(emb[nxt])
-            pos.add_(1)
-
-        def start(first):
-            x_in.copy_(emb[first])
-            pos.fill_(args.prompt)
-
-        first = prefill(ids)                                                # warm-up of the prefill lanes
+        first = dec.prefill(ids)                                            # warm-up of the prefill lanes
         torch.cuda.synchronize()
-        start(first)
+        dec.start(first, args.prompt)
         eager = []
         for _ in range(args.check_tokens):                                  # also warms the decode lanes up
-            step()
-            eager.append(tok.clone())
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
+            dec.step()
+            eager.append(dec.tok.clone())
         graph = None
         if not args.eager_decode:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                step()
-            start(first)
+            graph = dec.capture()
+            dec.start(first, args.prompt)
             agree = True
             for t in range(args.check_tokens):
                 graph.replay()
-                agree = agree and bool(torch.equal(tok, eager[t]))
+                agree = agree and bool(torch.equal(dec.tok, eager[t]))
             torch.cuda.synchronize()
             if not agree:
                 raise RuntimeError(f"decoder: graph replay and eager decoding disagree at batch {B}")
-        run_step = graph.replay if graph is not None else step
+        run_step = graph.replay if graph is not None else dec.step
 
         for L in layers:
             for lin in (L.qkv, L.o, L.gate_up, L.down):
@@ -534,12 +508,12 @@ def decoder(args):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.ttft_times):
-            first = prefill(ids)
+            first = dec.prefill(ids)
             torch.cuda.synchronize()
         ttft = (time.perf_counter() - t0) / args.ttft_times
         t0 = time.perf_counter()
-        first = prefill(ids)
-        start(first)
+        first = dec.prefill(ids)
+        dec.start(first, args.prompt)
         for _ in range(args.new_tokens - 1):
             run_step()
         torch.cuda.synchronize()
@@ -551,11 +525,11 @@ def decoder(args):
         kt = _KernelTimes()
         ops.set_tracer(kt)
         try:
-            first = prefill(ids)
+            first = dec.prefill(ids)
             conv_prefill, lib_prefill = kt.seconds()
             kt.pairs = []
-            start(first)
-            step()
+            dec.start(first, args.prompt)
+            dec.step()
             conv_step, lib_step = kt.seconds()
         finally:
             ops.set_tracer(None)
@@ -574,9 +548,7 @@ def decoder(args):
                                         for n, s in zip(("qkv", "o_proj", "gate_up", "down"), shapes)}})
         print(results[-1], file=sys.stderr, flush=True)
         del graph
-        for L in layers:
-            L.k_cache = L.v_cache = None
-        torch.cuda.empty_cache()
+        dec.free()
     return {"bench": "decoder", "layers": nl, "prompt": args.prompt, "new_tokens": args.new_tokens,
             "note": "random-init weights (one prepared layer cloned), fp16 SDPA attention in PyTorch over a static KV cache, "
                     + ("norms and SiLU * up in PyTorch" if args.torch_norm else "residual add + RMSNorm, and SiLU * up, each with the "
@@ -593,7 +565,6 @@ def main(argv=None):
     sub.add_parser("weightprep")
     sub.add_parser("blasref")
     sub.add_parser("actnorm")
-    sub.add_parser("mfmaceiling")
     d = sub.add_parser("decoder")
     d.add_argument("--lut", default=None)
     d.add_argument("--layers", type=int, default=32)
@@ -610,8 +581,7 @@ def main(argv=None):
     if args.cmd == "decoder" and args.lut is None:
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
-    ops.ensure_workspace()
-    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "mfmaceiling": mfmaceiling, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

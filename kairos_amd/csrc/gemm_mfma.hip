@@ -1025,16 +1025,12 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-// Caller-owned scratch for split-K partial sums, registered per host thread.  Optional: without it
-// (or when it is too small) no split is used.
-static thread_local void* g_workspace = nullptr;
-static thread_local size_t g_workspace_bytes = 0;
-extern "C" int kmi_gemm_set_workspace(void* ptr, size_t bytes) {
-    if (ptr && !kmi_aligned16(ptr)) return kmi_set_error(KMI_E_ALIGN, "kmi_gemm_set_workspace: pointer must be 16-byte aligned");
-    g_workspace = ptr;
-    g_workspace_bytes = ptr ? bytes : 0;
-    return KMI_OK;
-}
+// Scratch for split-K partial sums: every GEMM entry point takes a caller-owned device buffer (pointer and size)
+// and uses it only for the duration of the call's launches on the given stream.  Without one (NULL or too small
+// for two slices) no split is used.  Nothing about it is remembered between calls.
+struct Workspace { void* ptr; size_t bytes; };
+// Test and tuning hooks of the calling host thread (0 = automatic): they change speed and, for the fp16 lanes, the
+// order of the fp32 sums, never which entry point runs.
 static thread_local int g_force_splits = 0;
 extern "C" void kmi_gemm_force_splits(int splits) { g_force_splits = splits; }
 
@@ -1042,7 +1038,7 @@ extern "C" void kmi_gemm_force_splits(int splits) { g_force_splits = splits; }
 // round costs more than the idle CUs of the first), every split keeps at least eight 128-byte k-tiles,
 // and the partial sums fit the registered workspace.  Measured on MI355X: splitting 192 or 224 tiles in
 // two is 1.3-2x slower than running them as they are.
-static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
+static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles, const Workspace& ws) {
     const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     int s = 1;
     if (g_force_splits > 0) {
@@ -1054,8 +1050,8 @@ static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
         if (s > ktiles / 8) s = ktiles / 8;
     }
     const size_t per = (size_t)M * N * 4;
-    if (per == 0 || g_workspace == nullptr) return 1;
-    if ((size_t)s * per > g_workspace_bytes) s = (int)(g_workspace_bytes / per);
+    if (per == 0 || ws.ptr == nullptr) return 1;
+    if ((size_t)s * per > ws.bytes) s = (int)(ws.bytes / per);
     if (s > 1) {                                              // no empty split
         const int per_split = (ktiles + s - 1) / s;
         s = (ktiles + per_split - 1) / per_split;
@@ -1064,7 +1060,7 @@ static int pick_splits(int M, int N, int K, int BM, int BN, int ktiles) {
 }
 
 template <int KIND, int BM, int BN, bool TILED, int NS_ = 4>
-static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
+static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
@@ -1086,8 +1082,8 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, in
     const bool i8 = (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC);
     // units the kernels split K in: 128-byte k-tiles (register-staged) or 64-byte stages (direct)
     const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
-    a.splits = whole ? pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units) : 1;
-    a.partial = a.splits > 1 ? g_workspace : nullptr;
+    a.splits = whole ? pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units, ws) : 1;
+    a.partial = a.splits > 1 ? ws.ptr : nullptr;
     const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
@@ -1100,7 +1096,7 @@ static int launch_gemm(const GemmArgs& a_in, hipStream_t st, int n_begin = 0, in
 // Launch of the wave-private-weights kernel (W4A16, small M).  K is split over KH wave quartets inside the
 // workgroup and, when the tiles alone leave CUs idle, over workgroups as well (partials + reduce kernel).
 template <int BM, int KH = 2>
-static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
+static int launch_w4a16_wp(const GemmArgs& a_in, const Workspace& ws, hipStream_t st) {
     GemmArgs a = a_in;
     constexpr int PF = 4;
     constexpr size_t lds = (size_t)KH * (PF + 1) * BM * 128;
@@ -1119,15 +1115,15 @@ static int launch_w4a16_wp(const GemmArgs& a_in, hipStream_t st) {
     if (s > 8) s = 8;
     if (s > kt_all / 16) s = kt_all / 16;                       // at least 16 k-tiles (8 per quartet) per split
     const size_t per = (size_t)a.M * a.N * 4;
-    if (g_workspace == nullptr || per == 0) s = 1;
-    else if ((size_t)s * per > g_workspace_bytes) s = (int)(g_workspace_bytes / per);
+    if (ws.ptr == nullptr || per == 0) s = 1;
+    else if ((size_t)s * per > ws.bytes) s = (int)(ws.bytes / per);
     if (s < 1) s = 1;
     if (s > 1) {                                                 // whole quartet rounds per split, no empty split
         const int per_split = ((kt_all + s - 1) / s + KH - 1) / KH * KH;
         s = (kt_all + per_split - 1) / per_split;
     }
     a.splits = s;
-    a.partial = s > 1 ? g_workspace : nullptr;
+    a.partial = s > 1 ? ws.ptr : nullptr;
     hipLaunchKernelGGL(fn, dim3(tiles * s), dim3(256 * KH), lds, st, a);
     if (s > 1) {
         const long quads = (long)a.M * a.N / 4;
@@ -1199,23 +1195,23 @@ static WpChoice pick_wp(int M, int N, int K) {
 extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N, int K) { return pick_wp(M, N, K).rows; }
 
 template <int KIND, bool TILED>
-static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
+static int dispatch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t st, int force_tile) {
     const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N, (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC) ? (long)a.K : 0);
     if constexpr (KIND == KIND_W4A16) {
         // selectors 1032 / 1064 / 1128 force the wave-private-weights kernel with 32 / 64 / 128 rows per tile
-        if (tile == 1032) return launch_w4a16_wp<32>(a, st);
-        if (tile == 1064) return launch_w4a16_wp<64>(a, st);
-        if (tile == 1128) return launch_w4a16_wp<128>(a, st);
-        if (tile == 2032) return launch_w4a16_wp<32, 1>(a, st);      // 2xxx: one wave quartet per workgroup
-        if (tile == 2064) return launch_w4a16_wp<64, 1>(a, st);
-        if (tile == 2128) return launch_w4a16_wp<128, 1>(a, st);
+        if (tile == 1032) return launch_w4a16_wp<32>(a, ws, st);
+        if (tile == 1064) return launch_w4a16_wp<64>(a, ws, st);
+        if (tile == 1128) return launch_w4a16_wp<128>(a, ws, st);
+        if (tile == 2032) return launch_w4a16_wp<32, 1>(a, ws, st);      // 2xxx: one wave quartet per workgroup
+        if (tile == 2064) return launch_w4a16_wp<64, 1>(a, ws, st);
+        if (tile == 2128) return launch_w4a16_wp<128, 1>(a, ws, st);
         if (force_tile == 0) {
             const WpChoice c = pick_wp(a.M, a.N, a.K);
-            if (c.rows == 32) return launch_w4a16_wp<32>(a, st);
-            if (c.rows == 64 && c.quartets == 2) return launch_w4a16_wp<64>(a, st);
-            if (c.rows == 64) return launch_w4a16_wp<64, 1>(a, st);
-            if (c.rows == 128 && c.quartets == 2) return launch_w4a16_wp<128>(a, st);
-            if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, st);
+            if (c.rows == 32) return launch_w4a16_wp<32>(a, ws, st);
+            if (c.rows == 64 && c.quartets == 2) return launch_w4a16_wp<64>(a, ws, st);
+            if (c.rows == 64) return launch_w4a16_wp<64, 1>(a, ws, st);
+            if (c.rows == 128 && c.quartets == 2) return launch_w4a16_wp<128>(a, ws, st);
+            if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, ws, st);
         }
     }
     if (tile == 256 && force_tile == 0) {
@@ -1227,18 +1223,18 @@ static int dispatch_gemm(const GemmArgs& a, hipStream_t st, int force_tile) {
         const int tiles = TM * TN, rem = tiles % 256;
         const int head_cols = ((tiles - rem) / TM);          // column tiles that make up whole rounds
         if (tiles > 256 && rem > 0 && head_cols > 0 && (TN - head_cols) * TM <= 160) {
-            const int rc = launch_gemm<KIND, 256, 256, TILED>(a, st, 0, head_cols * 256);
+            const int rc = launch_gemm<KIND, 256, 256, TILED>(a, ws, st, 0, head_cols * 256);
             if (rc != KMI_OK) return rc;
-            return launch_gemm<KIND, 128, 128, TILED>(a, st, head_cols * 256, a.N - head_cols * 256);
+            return launch_gemm<KIND, 128, 128, TILED>(a, ws, st, head_cols * 256, a.N - head_cols * 256);
         }
     }
     switch (tile) {
-        case 256: return launch_gemm<KIND, 256, 256, TILED>(a, st);
+        case 256: return launch_gemm<KIND, 256, 256, TILED>(a, ws, st);
         case 192:                                        // 256 rows x 128 columns, three stages, two workgroups per CU
-            if constexpr (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16) return launch_gemm<KIND, 256, 128, TILED, 3>(a, st);
+            if constexpr (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16) return launch_gemm<KIND, 256, 128, TILED, 3>(a, ws, st);
             break;
-        case 128: return launch_gemm<KIND, 128, 128, TILED>(a, st);
-        case 64: return launch_gemm<KIND, 64, 128, TILED>(a, st);
+        case 128: return launch_gemm<KIND, 128, 128, TILED>(a, ws, st);
+        case 64: return launch_gemm<KIND, 64, 128, TILED>(a, ws, st);
     }
     return kmi_set_error(KMI_E_SHAPE, "gemm: unknown tile selector %d", tile);
 }
@@ -1257,16 +1253,27 @@ static int gemm_check(const char* fn, const GemmArgs& a, bool tiled) {
 static thread_local int g_force_tile = 0;
 extern "C" void kmi_gemm_force_tile(int tile) { g_force_tile = tile; }
 
+static int workspace_check(const char* fn, const void* workspace, size_t bytes, Workspace& ws) {
+    if (workspace && !kmi_aligned16(workspace)) return kmi_set_error(KMI_E_ALIGN, "%s: workspace must be 16-byte aligned", fn);
+    ws.ptr = const_cast<void*>(workspace);
+    ws.bytes = workspace ? bytes : 0;
+    return KMI_OK;
+}
+
 #define KMI_GEMM_BODY(NAME, KIND, TILED)                                      \
+    Workspace ws;                                                             \
     int rc = gemm_check(NAME, a, TILED);                                      \
     if (rc != KMI_OK) return rc;                                              \
+    rc = workspace_check(NAME, workspace, workspace_bytes, ws);               \
+    if (rc != KMI_OK) return rc;                                              \
     if (a.M == 0) return KMI_OK;                                              \
-    rc = dispatch_gemm<KIND, TILED>(a, static_cast<hipStream_t>(stream), g_force_tile); \
+    rc = dispatch_gemm<KIND, TILED>(a, ws, static_cast<hipStream_t>(stream), g_force_tile); \
     if (rc != KMI_OK) return rc;                                              \
     return kmi_check_launch(NAME);
 
 extern "C" int kmi_gemm_w4a16(void* out, const void* x, const void* qweight, const void* scales, const void* szeros,
-                              const void* bias, int M, int N, int K, int G, void* stream) {
+                              const void* bias, int M, int N, int K, int G, void* workspace, size_t workspace_bytes,
+                              void* stream) {
     if (G != 128) return kmi_set_error(KMI_E_GROUP, "kmi_gemm_w4a16: group size %d unsupported (128 only)", G);
     if (!scales || !szeros) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w4a16: NULL scale table");
     GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
@@ -1274,37 +1281,77 @@ extern "C" int kmi_gemm_w4a16(void* out, const void* x, const void* qweight, con
 }
 
 extern "C" int kmi_gemm_w8a16(void* out, const void* x, const void* w8, const void* wscales, const void* bias,
-                              int M, int N, int K, void* stream) {
+                              int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream) {
     if (!wscales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a16: NULL wscales");
     GemmArgs a{out, x, w8, nullptr, nullptr, (const half_t*)wscales, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a16", KIND_W8A16, false)
 }
 
 extern "C" int kmi_gemm_w8a8(void* out, const void* a8, const void* w8, const void* wscales, const void* ascales,
-                             const void* bias, int M, int N, int K, void* stream) {
+                             const void* bias, int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8: NULL scale vector");
     GemmArgs a{out, a8, w8, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8", KIND_W8A8, false)
 }
 
-extern "C" int kmi_gemm_w8a8_acc_i32(void* acc, const void* a8, const void* w8, int M, int N, int K, void* stream) {
+extern "C" int kmi_gemm_w8a8_acc_i32(void* acc, const void* a8, const void* w8, int M, int N, int K, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
     GemmArgs a{acc, a8, w8, nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8_acc_i32", KIND_W8A8_ACC, false)
 }
 
-extern "C" int kmi_gemm_f16(void* out, const void* x, const void* w16, const void* bias, int M, int N, int K, void* stream) {
+extern "C" int kmi_gemm_f16(void* out, const void* x, const void* w16, const void* bias, int M, int N, int K,
+                            void* workspace, size_t workspace_bytes, void* stream) {
     GemmArgs a{out, x, w16, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_f16", KIND_F16, false)
 }
 
 extern "C" int kmi_gemm_w8a8_tiled(void* out, const void* a8, const void* w8t, const void* wscales, const void* ascales,
-                                   const void* bias, int M, int N, int K, void* stream) {
+                                   const void* bias, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
     if (!wscales || !ascales) return kmi_set_error(KMI_E_NULL, "kmi_gemm_w8a8_tiled: NULL scale vector");
     GemmArgs a{out, a8, w8t, nullptr, nullptr, (const half_t*)wscales, (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_w8a8_tiled", KIND_W8A8, true)
 }
 
-extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, const void* bias, int M, int N, int K, void* stream) {
+extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, const void* bias, int M, int N, int K,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
     GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_f16_tiled", KIND_F16, true)
+}
+
+// Host-only query: the number of K splits a call of the given lane would use with a workspace of that size
+// (1 = none).  lane: 0 W4A16, 1 W8A16, 2 W8A8, 3 fp16; tiled as in the *_tiled entry points.
+extern "C" int kmi_gemm_splits_for(int lane, int M, int N, int K, size_t workspace_bytes) {
+    if (lane < 0 || lane > 3 || M <= 0 || N <= 0 || K <= 0 || (K & 127))
+        return kmi_set_error(KMI_E_SHAPE, "kmi_gemm_splits_for: bad arguments (lane=%d M=%d N=%d K=%d)", lane, M, N, K);
+    const Workspace ws{workspace_bytes ? reinterpret_cast<void*>(16) : nullptr, workspace_bytes};
+    const size_t per = (size_t)M * N * 4;
+    if (lane == 0) {
+        const WpChoice c = pick_wp(M, N, K);
+        if (c.rows) {                                         // mirrors launch_w4a16_wp
+            const int tiles = ((M + c.rows - 1) / c.rows) * ((N + 127) / 128), kt_all = K / 64, KH = c.quartets;
+            int s = g_force_splits > 0 ? g_force_splits : 256 / tiles;
+            if (s > 8) s = 8;
+            if (s > kt_all / 16) s = kt_all / 16;
+            if (ws.ptr == nullptr) s = 1;
+            else if ((size_t)s * per > ws.bytes) s = (int)(ws.bytes / per);
+            if (s < 1) s = 1;
+            if (s > 1) {
+                const int per_split = ((kt_all + s - 1) / s + KH - 1) / KH * KH;
+                s = (kt_all + per_split - 1) / per_split;
+            }
+            return s;
+        }
+    }
+    const bool i8 = lane == 2;
+    const int tile = g_force_tile > 0 ? g_force_tile : pick_tile(M, N, i8 ? (long)K : 0);
+    if (tile == 256 && g_force_tile == 0) {                   // mirrors the head/tail rule of dispatch_gemm: no split
+        const int TM = (M + 255) / 256, TN = (N + 255) / 256, tiles = TM * TN, rem = tiles % 256;
+        const int head_cols = (tiles - rem) / TM;
+        if (tiles > 256 && rem > 0 && head_cols > 0 && (TN - head_cols) * TM <= 160) return 1;
+    }
+    const int BM = tile == 64 ? 64 : tile == 128 ? 128 : 256, BN = (tile == 256) ? 256 : 128;
+    const int ktiles = (int)(((long)K * (i8 ? 1 : 2)) >> 7);
+    return pick_splits(M, N, K, BM, BN, ktiles, ws);
 }

@@ -9,8 +9,8 @@ exactly as serving stacks do with CUDA graphs.
 Capture rules this module enforces or relies on:
   * every kernel of the library launches on torch's current stream, so torch's stream capture records it;
   * the library records no memset nodes (none of its entry points clears memory);
-  * the temp cache and the split-K workspace are created BEFORE capture (they must not be allocated from
-    the graph's private pool, other graphs and eager calls share them);
+  * the temp cache and the capture stream's split-K scratch are created BEFORE capture, by warm-up calls on that
+    stream (they must not come from the graph's private pool: the temp cache is shared with eager calls);
   * the temp cache is invalidated right before capture, so every conversion the step needs is part of the
     graph, and after every replay, because the graph rewrites the cache behind the host-side tag's back;
   * inputs are copied into static buffers before each replay; outputs are the static tensors captured.
@@ -34,25 +34,28 @@ class GraphedCallable:
         if not torch.cuda.is_available():
             raise RuntimeError("GraphedCallable: needs a GPU")
         self._static_in = [x.clone() for x in example_inputs]
-        ops.ensure_workspace(device=self._static_in[0].device)
-        side = torch.cuda.Stream()                      # default priority
+        side = torch.cuda.Stream()                      # default priority; warm-up AND capture run on it
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            for _ in range(warmup):                     # sizes the temp cache, settles the LUT memo
-                fn(*self._static_in)
+            for _ in range(warmup):                     # sizes the temp cache, settles the LUT memo, creates this
+                fn(*self._static_in)                    # stream's split-K scratch outside the graph's memory pool
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self._caches = list(caches) if caches is not None else [default_cache()]
         self._invalidate()
+        for c in self._caches:
+            c.prepare_for_capture(self._static_in[0].device)
         self._graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self._graph):
+        with torch.cuda.graph(self._graph, stream=side):
             self._static_out = fn(*self._static_in)
         self._invalidate()
         self.replays = 0
 
     def _invalidate(self):
+        dev = self._static_in[0].device
         for c in self._caches:
             c.invalidate()
+            c.touch(dev)                                # the replay used the cache's buffer on the current stream
 
     def __call__(self, *inputs):
         if len(inputs) != len(self._static_in):

@@ -213,67 +213,103 @@ def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZ
     return out
 
 
+WORKSPACE_BYTES = 64 << 20
+_workspaces = {}                 # (device index, raw stream handle) -> uint8 tensor; never resized, never shared
+
+
+def workspace_for(device, stream=None):
+    """Split-K scratch of the calling stream: one fixed-size buffer per (device, stream), created on first use and
+    handed to every GEMM call as (pointer, bytes).  Two streams never share one, so concurrent GEMMs cannot race on
+    the partial sums; the size never changes, so a pointer baked into a captured graph stays valid for the life of
+    the process (drop_workspaces() is for tests only)."""
+    dev = torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if stream is None:
+        stream = _stream()
+    ws = _workspaces.get((idx, stream))
+    if ws is None:
+        ws = _workspaces[(idx, stream)] = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+    return ws
+
+
+def ensure_workspace(device="cuda", stream=None):
+    """Creates the calling (or given) stream's split-K scratch ahead of time, e.g. before a graph capture on it."""
+    return workspace_for(device, stream)
+
+
+def drop_workspaces():
+    """Forgets every scratch buffer (tests).  Not while a captured graph that used one is still alive."""
+    _workspaces.clear()
+
+
+def gemm_splits_for(lane, M, N, K, workspace_bytes=WORKSPACE_BYTES):
+    """K splits a GEMM call of `lane` ('w4a16', 'w8a16', 'w8a8', 'f16') would use with that much scratch (host only)."""
+    return _lib.check(_lib.load().kmi_gemm_splits_for({"w4a16": 0, "w8a16": 1, "w8a8": 2, "f16": 3}[lane], int(M), int(N),
+                                                      int(K), int(workspace_bytes)))
+
+
 def gemm_forward(x, qweight, scales, scaled_zeros, bias=None):
     """W4A16 MFMA GEMM for any m (gemm_cuda.cu:1126-1235).  Returns fp16 [*x.shape[:-1], N]."""
-    if _workspace is None:
-        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
     N, K = qweight.shape[0] * 4, qweight.shape[1]
     x2 = _flat2d(x)
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    st = _stream()
+    ws = workspace_for(x.device, st)
     _call("gemm_w4a16", x2.shape[0], N, K, _lib.load().kmi_gemm_w4a16, out.data_ptr(), x2.data_ptr(),
           qweight.data_ptr(), scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), x2.shape[0], N, K,
-          GROUP_SIZE, _stream())
+          GROUP_SIZE, ws.data_ptr(), ws.numel(), st)
     return out
 
 
 def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, tiled=False):
     """out_feats fp16 [M, N] <- int8 [M, K] x int8 [N, K] (w8a8_gemm_cuda.cu:909-954)."""
-    if _workspace is None:
-        ensure_workspace(device=in_feats.device)
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel"); _need(out_feats, torch.float16, "out_feats")
     M, K = in_feats.shape
     N = out_feats.shape[-1]
     fn = _lib.load().kmi_gemm_w8a8_tiled if tiled else _lib.load().kmi_gemm_w8a8
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
     _call("gemm_w8a8", M, N, K, fn, out_feats.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), wscales.data_ptr(),
-          ascales.data_ptr(), _ptr(bias), M, N, K, _stream())
+          ascales.data_ptr(), _ptr(bias), M, N, K, ws.data_ptr(), ws.numel(), st)
 
 
 def w8a8_gemm_acc_i32(in_feats, kernel, N):
     """Raw int32 accumulators [M, N] of the W8A8 product."""
-    if _workspace is None:
-        ensure_workspace(device=in_feats.device)
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel")
     M, K = in_feats.shape
     acc = torch.empty((M, N), dtype=torch.int32, device=in_feats.device)
-    _lib.check(_lib.load().kmi_gemm_w8a8_acc_i32(acc.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), M, N, K, _stream()))
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
+    _lib.check(_lib.load().kmi_gemm_w8a8_acc_i32(acc.data_ptr(), in_feats.data_ptr(), kernel.data_ptr(), M, N, K,
+                                                 ws.data_ptr(), ws.numel(), st))
     return acc
 
 
 def w8a16_gemm_forward(x, w8, wscales, N, bias=None):
     """fp16 [M, N] <- fp16 [M, K] x int8 [N, K] (row-major), per-channel scale in the epilogue."""
-    if _workspace is None:
-        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(w8, torch.int8, "w8")
     x2 = _flat2d(x)
     M, K = x2.shape
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
-    fn = _lib.load().kmi_gemm_w8a16
-    _call("gemm_w8a16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w8.data_ptr(), wscales.data_ptr(), _ptr(bias),
-          M, N, K, _stream())
+    st = _stream()
+    ws = workspace_for(x.device, st)
+    _call("gemm_w8a16", M, N, K, _lib.load().kmi_gemm_w8a16, out.data_ptr(), x2.data_ptr(), w8.data_ptr(),
+          wscales.data_ptr(), _ptr(bias), M, N, K, ws.data_ptr(), ws.numel(), st)
     return out
 
 
 def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
     """fp16 [M, N] <- fp16 [M, K] x fp16 [N, K] (`input @ tmp_weight.T`, dynamic_linear.py:163)."""
-    if _workspace is None:
-        ensure_workspace(device=x.device)
     _need(x, torch.float16, "x"); _need(w16, torch.float16, "w16")
     x2 = _flat2d(x)
     M, K = x2.shape
     out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
     fn = _lib.load().kmi_gemm_f16_tiled if tiled else _lib.load().kmi_gemm_f16
-    _call("gemm_f16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w16.data_ptr(), _ptr(bias), M, N, K, _stream())
+    st = _stream()
+    ws = workspace_for(x.device, st)
+    _call("gemm_f16", M, N, K, fn, out.data_ptr(), x2.data_ptr(), w16.data_ptr(), _ptr(bias), M, N, K,
+          ws.data_ptr(), ws.numel(), st)
     return out
 
 
@@ -287,29 +323,12 @@ def gemm_w4a16_wp_rows(M, N, K=4096):
     return _lib.load().kmi_gemm_w4a16_wp_rows(int(M), int(N), int(K))
 
 
-_workspace = None
-
-
-def ensure_workspace(nbytes=64 << 20, device="cuda"):
-    """Registers a persistent split-K scratch buffer (once per process) with the library."""
-    global _workspace
-    if _workspace is None or _workspace.numel() < nbytes:
-        _workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _lib.check(_lib.load().kmi_gemm_set_workspace(_workspace.data_ptr(), _workspace.numel()))
-    return _workspace
-
-
-def drop_workspace():
-    global _workspace
-    _lib.check(_lib.load().kmi_gemm_set_workspace(None, 0))
-    _workspace = None
-
-
 def force_gemm_splits(splits):
-    """Tuning hook: 0 = automatic, else the number of K splits (needs a registered workspace)."""
+    """Test hook of the calling thread: 0 = automatic, else the number of K splits."""
     _lib.load().kmi_gemm_force_splits(int(splits))
 
 
 def force_gemm_tile(tile):
-    """Tuning hook: 0 = automatic, else 64 / 128 / 256 (rows of the workgroup tile)."""
+    """Test hook of the calling thread: 0 = automatic, else 64 / 128 / 192 / 256 (and the 1xxx / 2xxx selectors of the
+    small-M W4A16 variant)."""
     _lib.load().kmi_gemm_force_tile(int(tile))

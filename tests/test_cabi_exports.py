@@ -44,11 +44,12 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 0, 64, 128, 128, None) == -4
     assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 65, 64, 128, 128, None) == -4
     assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 4, 60, 128, 128, None) == -2
-    assert lib.kmi_gemm_w8a8(16, 16, 16, 16, 16, None, 4, 64, 100, None) == -2
-    assert lib.kmi_gemm_w8a8(16, 16, 16, None, 16, None, 4, 64, 128, None) == -1
+    assert lib.kmi_gemm_w8a8(16, 16, 16, 16, 16, None, 4, 64, 100, None, 0, None) == -2
+    assert lib.kmi_gemm_w8a8(16, 16, 16, None, 16, None, 4, 64, 128, None, 0, None) == -1
     assert lib.kmi_quant_act_i8(16, 16, 16, 4, 12, None) == -2
     assert lib.kmi_quant_act_i8(16, 16, 16, 0, 128, None) == 0        # empty batch is a no-op
-    assert lib.kmi_gemm_f16(16, 16, 16, None, 0, 64, 128, None) == 0
+    assert lib.kmi_gemm_f16(16, 16, 16, None, 0, 64, 128, None, 0, None) == 0
+    assert lib.kmi_gemm_f16(16, 16, 16, None, 4, 64, 128, 8, 1024, None) == -5         # misaligned split-K scratch
     # fused preparation launch: same rules as its two halves
     assert lib.kmi_prep_w8a8(None, 0, 16, 16, 16, 4, 128, 128, 16, 16, 16, 2, None) == -1
     assert lib.kmi_prep_w8a8(16, 0, 16, 16, 16, 4, 128, 64, 16, 16, 16, 2, None) == -3
@@ -90,8 +91,29 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_silu_mul_quant_act(None, None, 8, 16, 2, 128, None) == -5
     assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 2, 100, None) == -2
     assert lib.kmi_silu_mul_quant_act(None, None, 16, 16, 0, 128, None) == 0
-    assert lib.kmi_probe_mfma(1, None, 16, 16, 4, 4, None) == -1 and lib.kmi_probe_mfma(1, 16, 16, 16, 0, 4, None) == -2
     assert lib.kmi_lut_get(None, 3) == -7
+
+
+def test_split_choice_depends_on_the_arguments_only(lib):
+    """The number of K splits is a function of shape and scratch size: the same on every host thread, whatever other
+    threads did before (there is no registration), 1 without scratch, never more than the scratch holds."""
+    import threading
+    MiB = 1 << 20
+    cases = [(0, 96, 1024, 4096), (0, 256, 4096, 14336), (2, 512, 4096, 14336), (2, 384, 4096, 4096), (3, 300, 4096, 4096),
+             (1, 128, 6144, 4096)]
+    main = [lib.kmi_gemm_splits_for(l, M, N, K, 64 * MiB) for l, M, N, K in cases]
+    assert all(s >= 1 for s in main) and any(s > 1 for s in main)
+    assert [lib.kmi_gemm_splits_for(l, M, N, K, 0) for l, M, N, K in cases] == [1] * len(cases)
+    for (l, M, N, K), s in zip(cases, main):
+        assert s == 1 or s * M * N * 4 <= 64 * MiB
+        small = lib.kmi_gemm_splits_for(l, M, N, K, 2 * M * N * 4)
+        assert small <= 2                                              # a buffer of two slices allows two splits at most
+    box = []
+    t = threading.Thread(target=lambda: box.append([lib.kmi_gemm_splits_for(l, M, N, K, 64 * MiB) for l, M, N, K in cases]))
+    t.start()
+    t.join()
+    assert box[0] == main
+    assert lib.kmi_gemm_splits_for(9, 16, 64, 128, 0) == -2 and lib.kmi_gemm_splits_for(0, 16, 64, 100, 0) == -2
 
 
 def test_lut_matches_oracle_on_reference_tables(lib, golden_dir):

@@ -145,3 +145,131 @@ def test_module_forward_full_size_rows(ops):
     x16 = O.synth_acts(16, K, seed=12)
     out16 = dl._forward(dev(x16)[None], 16, COMP_TYPE_NAME['w4a16_gemv'])[0]
     assert O.max_abs_rel(out16.cpu().numpy(), O.switched_forward(x16, p, COMP_TYPE_NAME['w4a16_gemv'])) < 1e-2
+
+
+def _exact_case(M, N, K, seed):
+    """Inputs whose product is exactly computable through every fp16 lane: integer weights q - 8 (tables s = 1,
+    z = -8), activations with sixteen entries of +-1, +-2, +-3 per row.  Every product and every partial sum is a
+    small integer (|sum| <= 16 * 3 * 8 = 384), exact in fp16 operands, fp32 accumulators and the fp16 output, in any
+    summation order.  Returns (q uint8 [N, K], a int8 [M, K], want fp16 [M, N])."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    a = np.zeros((M, K), dtype=np.int8)
+    # sixteen distinct columns per row: base + j * step, step < K / 16
+    idx = (rng.integers(0, K, size=(M, 1)) + rng.integers(1, K // 16, size=(M, 1)) * np.arange(16)[None, :]) % K
+    np.put_along_axis(a, idx, rng.choice(np.array([-3, -2, -1, 1, 2, 3], dtype=np.int8), size=(M, 16)), axis=1)
+    want = (a.astype(np.float32) @ (q.astype(np.float32) - 8.0).T).astype(np.float16)   # exact at every step
+    return q, a, want
+
+
+# every M x shape of the benchmark's large-M region; (lane, tile selector) pairs to run for each
+_FULL_F16 = [(M, N, K) for (N, K) in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)] for M in (1024, 2048, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", _FULL_F16)
+def test_f16_lanes_full_size_exact(ops, M, N, K):
+    """The fp16-output GEMM lanes at the benchmark's sizes, every kernel variant that can run them, bit for bit
+    against an exactly computable product: the register-staged kernel (W4A16 and W8A16; tiles 128 and 256 and the
+    automatic choice, which at 6144 columns and M = 4096 splits the launch into a 256-tile head and a 128-tile
+    tail), the wave-private W4A16 kernel (128-row tiles, one and two wave quartets, at the M it is selected for),
+    the direct-to-LDS fp16 kernel on row-major and on tiled weights (tiles 128, 192, 256, automatic), with a bias."""
+    q, a, want = _exact_case(M, N, K, seed=M + N + K)
+    qw = dev(O.pack_int_awq(q))
+    Gp = O.padded_groups(K)
+    ones = torch.ones((Gp, N), dtype=torch.float16, device="cuda")
+    x = dev(a.astype(np.float16))
+    bias_np = np.random.default_rng(N).integers(-64, 65, size=N).astype(np.float16)      # integer bias: still exact
+    bias = dev(bias_np)
+    want_b = (want.astype(np.float32) + bias_np.astype(np.float32)[None, :]).astype(np.float16)
+    want_t, want_bt = dev(want), dev(want_b)
+    w16 = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(w16, qw, ones, ones * -8.0, 128)
+    w16t = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(w16t, qw, ones, ones * -8.0, 128, tiled=True)
+    w8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(w8, qw, ones, ones * -8.0, 128)
+    half = torch.full((N,), 0.5, dtype=torch.float16, device="cuda")                     # W8A16 channel scale, exact
+    want_half = dev((want.astype(np.float32) * 0.5).astype(np.float16))
+
+    def same(got, ref, what):
+        torch.cuda.synchronize()
+        bad = (got.view(torch.int16) != ref.view(torch.int16)).sum().item()
+        assert bad == 0, f"{what}: {bad} of {got.numel()} elements differ (M={M} N={N} K={K})"
+
+    w4_tiles = [0, 128, 256] + ([1128, 2128] if M <= 1024 else [])
+    try:
+        for tile in w4_tiles:
+            ops.force_gemm_tile(tile)
+            same(ops.gemm_forward(x, qw, ones, ones * -8.0), want_t, f"w4a16 tile {tile}")
+        ops.force_gemm_tile(0)
+        same(ops.gemm_forward(x, qw, ones, ones * -8.0, bias=bias), want_bt, "w4a16 with bias")
+        for tile in (0, 128, 256):
+            ops.force_gemm_tile(tile)
+            same(ops.w8a16_gemm_forward(x, w8, half, N), want_half, f"w8a16 tile {tile}")
+        for tile in (0, 128, 192, 256):
+            ops.force_gemm_tile(tile)
+            same(ops.f16_gemm_forward(x, w16, N), want_t, f"f16 row-major tile {tile}")
+            same(ops.f16_gemm_forward(x, w16t, N, tiled=True), want_t, f"f16 tiled tile {tile}")
+        ops.force_gemm_tile(0)
+        same(ops.f16_gemm_forward(x, w16t, N, bias=bias, tiled=True), want_bt, "f16 tiled with bias")
+    finally:
+        ops.force_gemm_tile(0)
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 28672, 4096), (2048, 4096, 14336), (4096, 6144, 4096)])
+def test_f16_lanes_full_size_oracle_rows(ops, M, N, K):
+    """The same lanes on the benchmark's own data (prepared N(0, 0.02) weights, N(0, 1) activations with outlier
+    channels) against the oracle on sampled rows and a slice of columns: 2e-3 (bar 1e-2)."""
+    w = O.synth_weights(N, K, seed=10)
+    p = ops.prepare_weight(dev(w))
+    x = O.synth_acts(M, K, seed=11)
+    xd = dev(x)
+    rows = sample_rows(M, 6, N)
+    cols = slice(0, 1024)                                                      # 256 packed rows: the oracle's slice
+    qs = p["qweight"][: 1024 // 4].cpu().numpy()
+    sc, sz = p["scales"][:, cols].cpu().numpy(), p["scaled_zeros"][:, cols].cpu().numpy()
+    w16_ref = O.dequant_to_f16(qs, sc, sz)
+    ref = O.gemm_f16(x[rows], w16_ref)
+    ridx = torch.from_numpy(rows).cuda()
+    out4 = ops.gemm_forward(xd, p["qweight"], p["scales"], p["scaled_zeros"])
+    w16t = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(w16t, p["qweight"], p["scales"], p["scaled_zeros"], 128, tiled=True)
+    out16 = ops.f16_gemm_forward(xd, w16t, N, tiled=True)
+    w8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(w8, p["qweight"], p["scales_to8"], p["scaled_zeros_to8"], 128)
+    out816 = ops.w8a16_gemm_forward(xd, w8, p["scales_1"], N)
+    torch.cuda.synchronize()
+    assert O.max_abs_rel(out4[ridx][:, cols].cpu().numpy(), ref) < 2e-3
+    assert O.max_abs_rel(out16[ridx][:, cols].cpu().numpy(), ref) < 2e-3
+    w8_ref = O.dequant_to_i8(qs, p["scales_to8"][:, cols].cpu().numpy(), p["scaled_zeros_to8"][:, cols].cpu().numpy())
+    ref816 = O.gemm_w8a16(x[rows], w8_ref, p["scales_1"][cols].cpu().numpy())
+    assert O.max_abs_rel(out816[ridx][:, cols].cpu().numpy(), ref816) < 2e-3
+
+
+@pytest.mark.parametrize("N,K", [(3584, 18944), (4608, 3584)])
+def test_conversion_qwen_shapes_against_oracle(ops, N, K):
+    """int4 -> int8 / fp16, row-major and tiled, on the two Qwen2.5-7B shapes with padded table rows (K = 18944:
+    152 rows, 148 used; K = 3584: 32 rows, 28 used) and with N = 4608 = 36 strips of 128: every element against the
+    oracle, on prepared weights (whose tables the device preparation kernel wrote, zeros in the padded rows)."""
+    p = ops.prepare_weight(dev(O.synth_weights(N, K, seed=K)))
+    h = {k: v.cpu().numpy() for k, v in p.items()}
+    assert h["scales"].shape[0] == O.padded_groups(K) and not h["scales"][K // 128:].any()
+    want16 = O.dequant_to_f16(h["qweight"], h["scales"], h["scaled_zeros"])
+    want8 = O.dequant_to_i8(h["qweight"], h["scales_to8"], h["scaled_zeros_to8"])
+    for dtype, fn, tabs, want in ((torch.float16, ops.dequant_interleaved_int4_to_fp16, ("scales", "scaled_zeros"), want16),
+                                  (torch.int8, ops.dequant_interleaved_int4_to_int8, ("scales_to8", "scaled_zeros_to8"), want8)):
+        rows = torch.empty((N, K), dtype=dtype, device="cuda")
+        fn(rows, p["qweight"], p[tabs[0]], p[tabs[1]], 128)
+        tiled = torch.empty((N, K), dtype=dtype, device="cuda")
+        fn(tiled, p["qweight"], p[tabs[0]], p[tabs[1]], 128, tiled=True)
+        torch.cuda.synchronize()
+        bits = np.uint16 if dtype is torch.float16 else np.uint8
+        assert np.array_equal(rows.cpu().numpy().view(bits), want.view(bits))
+        assert np.array_equal(ops.untile(tiled, N, K).cpu().numpy().view(bits), want.view(bits))
+    # the fused preparation launch writes the same int8 weight (and quantises a few tokens beside it)
+    x = dev(O.synth_acts(5, K, seed=3))
+    w8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    a8 = torch.empty((5, K), dtype=torch.int8, device="cuda")
+    sx = torch.empty((5,), dtype=torch.float16, device="cuda")
+    ops.prep_w8a8(w8, p["qweight"], p["scales_to8"], p["scaled_zeros_to8"], a8, x, sx, 128, tiled=True)
+    assert np.array_equal(ops.untile(w8, N, K).cpu().numpy(), want8)

@@ -266,3 +266,122 @@ def test_quantized_llama_matches_dequantised_model(gpu):
                 assert err < tol, (T, err)
     finally:
         DynamicLinear.prof = old
+
+
+def test_split_k_result_does_not_depend_on_the_calling_thread(gpu):
+    """The split-K scratch travels with every call, so a GEMM issued from a second host thread splits exactly as
+    on the main thread and returns the same bits (fp16 lanes: same fp32 summation order)."""
+    import threading
+    from kairos_amd import ops
+    N, K, M = 1024, 4096, 96
+    p = ops.prepare_weight(torch.from_numpy(O.synth_weights(N, K, seed=4)).cuda())
+    x = torch.from_numpy(O.synth_acts(M, K, seed=5)).cuda()
+    assert ops.gemm_splits_for("w4a16", M, N, K) > 1 and ops.gemm_splits_for("w4a16", M, N, K, 0) == 1
+    main = ops.gemm_forward(x, p["qweight"], p["scales"], p["scaled_zeros"])
+    torch.cuda.synchronize()
+    box = {}
+
+    def worker():
+        torch.cuda.set_device(0)
+        box["splits"] = ops.gemm_splits_for("w4a16", M, N, K)
+        box["out"] = ops.gemm_forward(x, p["qweight"], p["scales"], p["scaled_zeros"])
+        torch.cuda.synchronize()
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert box["splits"] == ops.gemm_splits_for("w4a16", M, N, K)
+    assert torch.equal(box["out"].view(torch.int16), main.view(torch.int16))
+    # two streams never share a scratch buffer
+    s2 = torch.cuda.Stream()
+    with torch.cuda.stream(s2):
+        other = ops.gemm_forward(x, p["qweight"], p["scales"], p["scaled_zeros"])
+        ws2 = ops.workspace_for(x.device)
+    s2.synchronize()
+    assert ws2.data_ptr() != ops.workspace_for(x.device).data_ptr()
+    assert torch.equal(other.view(torch.int16), main.view(torch.int16))
+
+
+def test_decoder_harness_two_layers(gpu):
+    """The end-to-end decoder harness (GQA attention over a static KV cache, matched norm and SiLU operators, every
+    linear a LUT-switched DynamicLinear, decode step replayed from a HIP graph) at reduced width, two layers:
+    prefill and decode logits against the same stack computing with the oracle's dequantised fp16 weights in
+    PyTorch, and graph-replayed tokens against eagerly generated ones."""
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.perf_profiler import Profiler
+    from kairos_amd.bench_extra import Decoder
+    dev = torch.device("cuda:0")
+    hidden, heads, kv, mlp, vocab = 1024, 8, 2, 2048, 2048
+    d = hidden // heads
+    shapes = [((heads + 2 * kv) * d, hidden), (hidden, hidden), (2 * mlp, hidden), (hidden, mlp)]
+    prof = Profiler(shapes)
+    for s in shapes:
+        for r, name in [(16, 'w4a16_gemv'), (128, 'w4a16_gemm'), (1 << 20, 'w8a8')]:
+            prof.record_best_comp(s, r, name)
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+
+    class Dense(torch.nn.Module):                       # the comparison stack's linear: fp16 matmul on dequantised weights
+        def __init__(self, w16):
+            super().__init__()
+            self.w = w16
+
+        def forward(self, x):
+            return x @ self.w.T
+
+    try:
+        quant, dense = [], []
+        for l in range(2):
+            ql, dl_ = [], []
+            for i, (N, K) in enumerate(shapes):
+                w = O.synth_weights(N, K, seed=100 + 10 * l + i) * np.float16(2.0)
+                lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16)
+                with torch.no_grad():
+                    lin.weight.copy_(torch.from_numpy(w))
+                ql.append(DynamicLinear.from_module(lin.cuda(), "cuda"))
+                p = O.prepare_weights(w)
+                dl_.append(Dense(torch.from_numpy(O.dequant_to_f16(p["qweight"], p["scales"], p["scaled_zeros"])).cuda()))
+            quant.append(ql)
+            dense.append(dl_)
+        t_max = 160
+        dec = Decoder(quant, dev, hidden, heads, kv, vocab, matched=True, t_max=t_max, seed=1)
+        ref = Decoder(dense, dev, hidden, heads, kv, vocab, matched=False, t_max=t_max, seed=1)
+        assert torch.equal(dec.emb, ref.emb) and torch.equal(dec.head, ref.head)
+        B = 2
+
+        def rel(a, b):
+            return ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+
+        for prompt, tol in ((24, 1e-2), (128, 6e-2)):   # 48 tokens: W4A16 GEMM prefill; 256 tokens: W8A8 prefill
+            ids = torch.randint(0, vocab, (B, prompt), device=dev, generator=torch.Generator(device=dev).manual_seed(prompt))
+            dec.alloc(B)
+            ref.alloc(B)
+            got, want = dec.prefill_logits(ids), ref.prefill_logits(ids)
+            assert torch.isfinite(got).all() and rel(got, want) < tol, (prompt, rel(got, want))
+            lanes = {prof.get_comp_type(s, B * prompt) for s in shapes}
+            assert lanes == ({0} if prompt == 24 else {2})
+            if prompt != 24:
+                continue
+            # decode: the small-M lane on the quantised stack; both stacks continue from the comparison stack's token
+            first = want.argmax(-1)
+            dec.start(first, prompt)
+            ref.start(first, prompt)
+            eager = []
+            for t in range(6):
+                dec.step()
+                ref.step()
+                assert rel(dec.logits, ref.logits) < 2e-2, (t, rel(dec.logits, ref.logits))
+                eager.append((dec.tok.clone(), dec.logits.clone()))
+                ref.x_in.copy_(dec.x_in)                # keep the two sequences on the same tokens
+            graph = dec.capture()
+            dec.prefill_logits(ids)                     # the capture's warm-up step wrote the cache: refill it
+            dec.start(first, prompt)
+            for t in range(6):
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(dec.tok, eager[t][0]), f"token {t}: graph replay and eager decoding disagree"
+                assert torch.equal(dec.logits.view(torch.int16), eager[t][1].view(torch.int16))
+            dec.free()
+            ref.free()
+    finally:
+        DynamicLinear.prof = old

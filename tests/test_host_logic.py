@@ -143,6 +143,94 @@ def test_temp_cache_is_bounded_and_reuses():
     assert c.capacity <= 1024
 
 
+class _FakeStreams:
+    """Stand-ins for the stream queries of kairos_amd.temp_cache, so that its capture and multi-stream rules can be
+    exercised without a GPU: `current` names the stream, `capturing` says whether it records a graph."""
+
+    def __init__(self, monkeypatch):
+        from kairos_amd import temp_cache as tc
+        self.current, self.capturing, self.orders = "s0", False, []
+        monkeypatch.setattr(tc, "_is_capturing", lambda device: self.capturing)
+        monkeypatch.setattr(tc, "_current_stream", lambda device: self.current)
+        monkeypatch.setattr(tc, "_order_after", lambda stream, earlier: self.orders.append((stream, earlier)))
+
+
+def test_temp_cache_never_bakes_a_hit_into_a_graph(monkeypatch):
+    """A request made during graph capture is a miss (the conversion must be recorded: at replay time the buffer
+    holds whatever ran last) and clears the tag, so the next eager request converts as well."""
+    from kairos_amd.temp_cache import TempCache
+    st = _FakeStreams(monkeypatch)
+    c = TempCache()
+    a, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert not hit and c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]          # eager: second call hits
+    st.capturing = True
+    b, hit = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert not hit and b.data_ptr() == a.data_ptr()                            # same buffer, but converted in the graph
+    assert not c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]                   # still capturing: never a hit
+    with pytest.raises(RuntimeError, match="eagerly"):                         # growth inside a capture is refused
+        c.get(2, 'f16', (64, 64), torch.float16, 'cpu')
+    st.capturing = False
+    assert not c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]                   # the capture left the tag cleared
+    assert c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]
+
+
+def test_temp_cache_keeps_a_captured_buffer_alive_when_it_grows(monkeypatch):
+    from kairos_amd.temp_cache import TempCache
+    st = _FakeStreams(monkeypatch)
+    c = TempCache()
+    small, _ = c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    st.capturing = True
+    c.get(1, 'i8', (4, 64), torch.int8, 'cpu')                                 # a graph records this address
+    st.capturing = False
+    storage = small.untyped_storage().data_ptr()
+    big, hit = c.get(2, 'f16', (64, 64), torch.float16, 'cpu')                 # eager growth afterwards
+    assert not hit and big.untyped_storage().data_ptr() != storage
+    assert [b.untyped_storage().data_ptr() for b in c._retired] == [storage]   # still referenced: not freed, not reused
+    c2 = TempCache()
+    c2.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    c2.get(2, 'f16', (64, 64), torch.float16, 'cpu')                           # no capture in between: nothing kept aside
+    assert c2._retired == []
+
+
+def test_temp_cache_orders_requests_from_different_streams(monkeypatch):
+    """The buffer handed out on stream s1 after a use on s0 is ordered behind s0's queue (the earlier conversion and
+    the GEMM that reads it), for hits and misses alike; requests on one stream need no event."""
+    from kairos_amd.temp_cache import ResidentCache, TempCache
+    st = _FakeStreams(monkeypatch)
+    c = TempCache()
+    c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    c.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    assert st.orders == []
+    st.current = "s1"
+    assert c.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1] and st.orders == [("s1", "s0")]     # a safe hit
+    c.get(2, 'i8', (4, 64), torch.int8, 'cpu')
+    assert st.orders == [("s1", "s0")]
+    st.current = "s0"
+    assert not c.get(3, 'i8', (4, 64), torch.int8, 'cpu')[1] and st.orders[-1] == ("s0", "s1")
+    # a graph replay on s2 uses the buffer behind the cache's back: touch() makes the next request wait for it
+    st.current = "s2"
+    c.touch('cpu')
+    st.current = "s0"
+    c.get(3, 'i8', (4, 64), torch.int8, 'cpu')
+    assert st.orders[-2:] == [("s2", "s0"), ("s0", "s2")]
+    # the many-entry cache keeps one order per copy and converts inside captures without keeping anything
+    st.orders.clear()
+    r = ResidentCache(4096)
+    monkeypatch.setattr(torch.Tensor, "record_stream", lambda self, s: None, raising=False)
+    r.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    st.current = "s1"
+    assert r.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1] and st.orders == [("s1", "s0")]
+    st.capturing = True
+    with pytest.raises(RuntimeError, match="prepare_for_capture"):
+        r.get(1, 'i8', (4, 64), torch.int8, 'cpu')
+    st.capturing = False
+    r.prepare_for_capture('cpu')
+    st.capturing = True
+    assert not r.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1] and not r.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]
+    st.capturing = False
+    assert r.get(1, 'i8', (4, 64), torch.int8, 'cpu')[1]                       # the resident copy was left alone
+
+
 def test_committed_mi355x_tables_load_and_have_three_regimes():
     """Every table shipped under kairos_amd/prof/ has the reference's file format and the small-M / mid-M /
     large-M structure (same schema as the reference's prof_llama / prof_qwen files)."""
