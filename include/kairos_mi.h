@@ -196,6 +196,19 @@ int kmi_gemm_w8a8_tiled(void* out_f16, const void* a8, const void* w8_tiled, con
 int kmi_gemm_f16_tiled(void* out_f16, const void* x_f16, const void* w16_tiled, const void* bias,
                        int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 
+/* kmi_gemm_w4a16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no counterpart in the reference.  Same kernels, same results, but the split-K
+ * partial sums go to a 16 MiB array that is part of the library's code object (one copy per GPU, held until the
+ * process ends) instead of a caller-owned workspace; the call allocates and frees nothing.  Limits: M*N <=
+ * KMI_NOALLOC_MAX_OUTPUTS (KMI_E_M_RANGE beyond); the stream must belong to the current device; the first call on a
+ * device looks the array's address up and must not run inside a graph capture.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (different streams, or replays of graphs that contain one) race on it.
+ * Nothing needs clearing between calls (every partial sum that is read was written by the same call). */
+#define KMI_NOALLOC_MAX_OUTPUTS (512 * 1024)
+#define KMI_NOALLOC_MAX_DEVICES 64
+int kmi_gemm_w4a16_noalloc(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                           const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
+
 /* Host-only queries of the automatic choices (no GPU work).
  * kmi_gemm_pick_tile: the workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns) of the W8A8 lane for an
  *   M x N x K product.  With the 256 tile the library may run the columns of a thin last round of tiles with the 128

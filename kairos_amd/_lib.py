@@ -33,6 +33,7 @@ SIGNATURES = {
     "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     # GEMMs end with (workspace pointer, workspace bytes, stream)
     "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w4a16_noalloc": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "kmi_gemm_w8a16": [_P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w8a8": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w8a8_acc_i32": [_P, _P, _P, _I, _I, _I, _P, _Z, _P],

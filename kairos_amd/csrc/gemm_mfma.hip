@@ -15,6 +15,7 @@
 // W4A16 products of up to ~1000 rows run gemm_w4a16_wp_kernel instead (weights decoded in registers by the wave
 // that owns their columns, never written to LDS); the host side at the end of the file picks kernel and tile.
 #include "kmi_common.h"
+#include <mutex>
 #include <type_traits>
 
 enum { KIND_F16 = 0, KIND_W4A16 = 1, KIND_W8A16 = 2, KIND_W8A8 = 3, KIND_W8A8_ACC = 4 };
@@ -1318,6 +1319,52 @@ extern "C" int kmi_gemm_f16_tiled(void* out, const void* x, const void* w16t, co
                                   void* workspace, size_t workspace_bytes, void* stream) {
     GemmArgs a{out, x, w16t, nullptr, nullptr, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
     KMI_GEMM_BODY("kmi_gemm_f16_tiled", KIND_F16, true)
+}
+
+// ---- the W4A16 GEMM for callers that cannot allocate --------------------------------------------------------------
+// Same kernels as kmi_gemm_w4a16; the split-K partial sums live in a file-scope device array instead of a buffer the
+// caller brings.  Every GPU the library's code object is loaded on holds its own copy of the array until the process
+// ends, at its own address: that address is looked up once per device and is what the kernels receive.
+#define KMI_NOALLOC_SCRATCH_BYTES (16u << 20)
+static __device__ __align__(256) unsigned char scratch[KMI_NOALLOC_SCRATCH_BYTES];
+static void* g_scratch_ptr[KMI_NOALLOC_MAX_DEVICES] = {};      // device address of `scratch`, per device ordinal
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(const char* fn, void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= KMI_NOALLOC_MAX_DEVICES)
+        return kmi_set_error(KMI_E_LAUNCH, "%s: cannot identify the current device (ordinal %d)", fn, dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return kmi_set_error(KMI_E_LAUNCH, "%s: hipGetSymbolAddress failed on device %d: %s", fn, dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return KMI_OK;
+}
+
+extern "C" int kmi_gemm_w4a16_noalloc(void* out, const void* x, const void* qweight, const void* scales, const void* szeros,
+                                      const void* bias, int M, int N, int K, int G, void* stream) {
+    const char* fn = "kmi_gemm_w4a16_noalloc";
+    if (G != 128) return kmi_set_error(KMI_E_GROUP, "%s: group size %d unsupported (128 only)", fn, G);
+    if (!scales || !szeros) return kmi_set_error(KMI_E_NULL, "%s: NULL scale table", fn);
+    GemmArgs a{out, x, qweight, (const half_t*)scales, (const half_t*)szeros, nullptr, nullptr, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
+    int rc = gemm_check(fn, a, false);
+    if (rc != KMI_OK) return rc;
+    if ((long)M * N > KMI_NOALLOC_MAX_OUTPUTS)
+        return kmi_set_error(KMI_E_M_RANGE, "%s: M*N = %ld outputs exceed the %d this entry point's built-in scratch serves "
+                             "(use kmi_gemm_w4a16 with a workspace)", fn, (long)M * N, KMI_NOALLOC_MAX_OUTPUTS);
+    if (a.M == 0) return KMI_OK;
+    static_assert((size_t)KMI_NOALLOC_MAX_OUTPUTS * 4 * 8 <= KMI_NOALLOC_SCRATCH_BYTES, "eight fp32 slices of the largest output");
+    Workspace ws{nullptr, KMI_NOALLOC_SCRATCH_BYTES};
+    rc = scratch_of_current_device(fn, &ws.ptr);
+    if (rc != KMI_OK) return rc;
+    rc = dispatch_gemm<KIND_W4A16, false>(a, ws, static_cast<hipStream_t>(stream), g_force_tile);
+    if (rc != KMI_OK) return rc;
+    return kmi_check_launch(fn);
 }
 
 // Host-only query: the number of K splits a call of the given lane would use with a workspace of that size
