@@ -25,7 +25,7 @@ sys.path.insert(0, ROOT)
 LAYER = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)]
 M_GRID = [1 << i for i in range(13)]
 PEAK = {"hbm": 8.0e12, "f16": 2.5e15, "i8": 5.0e15}       # MI355X published: HBM3E B/s, dense MFMA op/s
-LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x")
+LUT_DIR = os.path.join(ROOT, "kairos_amd", "prof", "llama3_8b_mi355x_v2")     # version-2 id table: adds the W4A8 lane
 # HBM<->L2 bytes per call of the dominant kernel: written by `python -m kairos_amd.traffic` from two rocprofv3 counter
 # runs of this script (--only-label), stamped with a hash of the kernel sources; ignored once the sources change.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_llama3_8b_traffic.json")
@@ -61,6 +61,8 @@ def algorithmic(kernel, M, N, K):
         return algorithmic("cvt_i4_to_i8", 0, N, K)[0] + algorithmic("quant_act_i8", M, 0, K)[0], 0, None
     if kernel == "gemm_w8a8":
         return M * K + N * K + 2 * N + 2 * M + 2 * M * N, 2 * M * N * K, "i8"
+    if kernel == "gemm_w4a8":                         # int8 activations, packed int4 weights + their two tables
+        return M * K + N * K // 2 + 4 * (K // G) * N + 2 * N + 2 * M + 2 * M * N, 2 * M * N * K, "i8"
     if kernel == "gemm_w8a16":
         return 2 * M * K + N * K + 2 * N + 2 * M * N, 2 * M * N * K, "f16"
     if kernel == "gemm_f16":
@@ -87,6 +89,8 @@ class Tracer:
         label = name
         if name == "gemm_w4a16" and self.ops.gemm_w4a16_wp_rows(M, N, K):
             label = f"{name}[wp{self.ops.gemm_w4a16_wp_rows(M, N, K)}]"
+        elif name == "gemm_w4a8":
+            label = f"{name}[{self.ops.gemm_w4a8_tile_for(M, N, K)}]"
         elif name.startswith("gemm_"):
             label = f"{name}[{self.ops.gemm_tile_for(M, N, K)}]"
         ev = self.torch.cuda.Event(enable_timing=True)
@@ -229,8 +233,8 @@ def main():
         print("bench.py: no GPU visible; the HIP library is the only compute path", file=sys.stderr)
         sys.exit(3)
     from kairos_amd import ops
-    from kairos_amd.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
-    from kairos_amd.perf_profiler import Profiler
+    from kairos_amd.dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear
+    from kairos_amd.perf_profiler_v2 import Profiler
     from kairos_amd import traffic
 
     dev = torch.device("cuda:0")
@@ -292,8 +296,8 @@ def main():
         for M in M_GRID:
             for li, (_n, N, K) in enumerate(LAYER):
                 lane = names[prof.get_comp_type((N, K), M)]
-                kern = {"w4a16_gemv": "gemv_w4a16", "w4a16_gemm": "gemm_w4a16", "w8a8": "gemm_w8a8",
-                        "w8a16_gemm": "gemm_w8a16", "fp16": "gemm_f16"}[lane]
+                kern = {"w4a16_gemv": "gemv_w4a16", "w4a16_gemm": "gemm_w4a16", "w8a8": "gemm_w8a8", "w4a16_marlin": "gemm_w4a16",
+                        "w8a16_gemm": "gemm_w8a16", "fp16": "gemm_f16", "w4a8_qserve": "gemm_w4a8"}[lane]
                 probe = Tracer(torch, ops)
                 probe.begin(kern, M, N, K)
                 if probe._cur[0] == args.only_label:
@@ -407,7 +411,7 @@ def main():
 
     sweep = []
     if not args.no_sweep:
-        lanes = ["w4a16_gemv", "w4a16_gemm", "w8a16_gemm", "w8a8", "fp16"]
+        lanes = ["w4a16_gemv", "w4a16_gemm", "w8a16_gemm", "w8a8", "w4a8_qserve", "fp16"]
         for li, (lname, N, K) in enumerate(LAYER):
             for M in M_GRID:
                 for lane in lanes:
@@ -420,7 +424,7 @@ def main():
                         layers[li][i % args.copies]._forward(acts[(M, K)], M, cid)
                     us = time_calls(call, n)
                     main_kernel = {"w4a16_gemv": "gemv_w4a16", "w4a16_gemm": "gemm_w4a16", "w8a16_gemm": "gemm_w8a16",
-                                   "w8a8": "gemm_w8a8", "fp16": "gemm_f16"}[lane]
+                                   "w8a8": "gemm_w8a8", "w4a8_qserve": "gemm_w4a8", "fp16": "gemm_f16"}[lane]
                     ideal, bnd = roofline_time(main_kernel, M, N, K)
                     b, f, _dt = algorithmic(main_kernel, M, N, K)
                     sweep.append({"shape": lname, "N": N, "K": K, "M": M, "lane": lane, "us": round(us, 2),
@@ -448,7 +452,7 @@ def main():
         rows = [s for s in sweep if pred(s)]
         return max(rows, key=lambda s: s["roofline_frac"]) if rows else None
     small = best(lambda s: s["M"] <= 16 and s["lane"] == "w4a16_gemv")
-    large = best(lambda s: s["M"] >= 1024 and s["lane"] in ("w8a8", "w4a16_gemm", "fp16", "w8a16_gemm"))
+    large = best(lambda s: s["M"] >= 1024 and s["lane"] in ("w8a8", "w4a8_qserve", "w4a16_gemm", "fp16", "w8a16_gemm"))
 
     # the GPU on the CPU leg's sample: config 1 through the small-M lane
     cfg1_us = time_calls(lambda i=0: layers[1][i % args.copies]._forward(acts[(16, 4096)], 16, COMP_TYPE_NAME["w4a16_gemv"]), 50)

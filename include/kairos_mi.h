@@ -184,6 +184,24 @@ int kmi_gemm_w8a8(void* out_f16, const void* a8, const void* w8, const void* wsc
 int kmi_gemm_w8a8_acc_i32(void* acc_i32, const void* a8, const void* w8, int M, int N, int K,
                           void* workspace, size_t workspace_bytes, void* stream);
 
+/* W4A8: the W8A8 product computed from the resident packed int4 weight, with no converted copy:
+ *   acc = a8 . W8^T,  W8[n,k] = (int8) fma_f16(q[n,k], scales_to8[k/G,n], scaled_zeros_to8[k/G,n])  (what kmi_cvt_i4_to_i8 writes),
+ *   out = fp16(float(acc) * (float(wscales[n]) * float(ascales[m]))) (+bias),
+ * so accumulators and outputs equal kmi_cvt_i4_to_i8 + kmi_gemm_w8a8 bit for bit.  It takes the place of the
+ * version-2 candidate `w4a8_qserve` (kairos/dynamic_linear_v2.py:161-179: trans_layout_c16_to_c8_awq + a third-party
+ * int4 x int8 GEMM with its own second-level quantiser): same operand precisions, weights decoded inside the GEMM.
+ * kmi_gemm_w4a8_acc_i32 writes the raw int32 accumulators [M, N] (bit-exact tier).  kmi_gemm_w4a8_pick_tile: host-only,
+ * the tile selector the call would use (128 = 128 x 128, 192 = 256 rows x 128 columns, 256 = 256 x 256, 448 = 256 x 256
+ * tiles in whole rounds over the CUs and the remaining columns as 256 x 128 tiles in a second launch on the same stream);
+ * kmi_gemm_force_tile accepts the same selectors for this lane. */
+int kmi_gemm_w4a8(void* out_f16, const void* a8, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
+                  const void* wscales_f16, const void* ascales_f16, const void* bias, int M, int N, int K, int G,
+                  void* workspace, size_t workspace_bytes, void* stream);
+int kmi_gemm_w4a8_acc_i32(void* acc_i32, const void* a8, const void* qweight, const void* scales_to8,
+                          const void* scaled_zeros_to8, int M, int N, int K, int G,
+                          void* workspace, size_t workspace_bytes, void* stream);
+int kmi_gemm_w4a8_pick_tile(int M, int N, int K);
+
 /* FP16: out = x . w16^T (+bias), fp32 accumulation.  Replaces `input @ tmp_weight.T`
  * (kairos/dynamic_linear.py:163). */
 int kmi_gemm_f16(void* out_f16, const void* x_f16, const void* w16, const void* bias,

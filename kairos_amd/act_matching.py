@@ -12,7 +12,7 @@ projection does the same (`kmi_silu_mul_quant_act`).  A `MatchedActivation` carr
 import torch
 
 from . import ops
-from .dynamic_linear import _W8A8, DynamicLinear
+from .dynamic_linear import _W4A8, _W8A8, DynamicLinear
 
 
 class MatchedActivation:
@@ -28,11 +28,11 @@ class MatchedActivation:
 
 
 def _formats_for(consumers, m):
-    """(want_f16, want_i8) for m tokens: int8 if a consumer's lane is W8A8, fp16 if one is anything else."""
+    """(want_f16, want_i8) for m tokens: int8 if a consumer's lane takes int8 activations (W8A8, W4A8), fp16 if one is anything else."""
     want_f16 = want_i8 = False
     for lin in consumers:
         comp = type(lin).prof.get_comp_type(lin.shape, m) if isinstance(lin, DynamicLinear) else None
-        if comp == _W8A8:
+        if comp in (_W8A8, _W4A8):
             want_i8 = True
         else:
             want_f16 = True

@@ -8,6 +8,9 @@ the offline-profiled interval table of this layer's shape and runs one of the HI
     w8a8       (2)  int4->int8 conversion + per-token int8 activations + int8 MFMA GEMM
     w8a16_*  (3,4)  int4->int8 conversion + fp16 activations, fp16 MFMA GEMM (declared but unused upstream)
     fp16       (5)  int4->fp16 conversion + fp16 MFMA GEMM
+    w4a16 alt  (6)  version-2 tables only: the W4A16 MFMA GEMM again (one W4A16 GEMM exists here)
+    w4a8       (7)  version-2 tables only: per-token int8 activations x int4 weights decoded inside the int8 MFMA
+                    GEMM; same results as w8a8, no converted copy                  kmi_gemm_w4a8
 
 Same constructor, class attribute `prof`, `from_module`, `forward`, `_forward` and tensor attributes
 as the reference module.
@@ -24,6 +27,7 @@ COMP_TYPE_NAME = {'w4a16_gemm': 0, 'w4a16_gemv': 1, 'w8a8': 2,
                   'w8a16_gemm': 3, 'w8a16_gemv': 4, 'fp16': 5}
 
 _W4A16_GEMM, _W4A16_GEMV, _W8A8, _W8A16_GEMM, _W8A16_GEMV, _FP16 = 0, 1, 2, 3, 4, 5
+_W4A16_ALT, _W4A8 = 6, 7          # ids of the version-2 table (kairos/dynamic_linear_v2.py:11-13)
 _uids = itertools.count(1)
 RESIDENT_KEYS = ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1")
 
@@ -150,6 +154,8 @@ class DynamicLinear(torch.nn.Module):
         if not isinstance(input, torch.Tensor):              # a MatchedActivation from the operator in front
             if self.comp_type == _W8A8 and input.int_x is not None:
                 return self._w8a8(None, input.int_x.reshape(-1, K), input.scale_x).reshape(*shape[:-1], -1)
+            if self.comp_type == _W4A8 and input.int_x is not None:
+                return self._w4a8(None, input.int_x.reshape(-1, K), input.scale_x).reshape(*shape[:-1], -1)
             if input.f16 is None:
                 raise ValueError("the matched activation holds no fp16 form, but this layer's lane for "
                                  f"{m} tokens (id {self.comp_type}) needs one")
@@ -201,6 +207,19 @@ class DynamicLinear(torch.nn.Module):
         ops.w8a8_gemm_forward(int_x, w8, self.scales_1, scale_x, out, bias=self.bias, tiled=tiled)
         return out
 
+    def _w4a8(self, x, int_x, scale_x):
+        """The W4A8 lane on fp16 activations x [m, K], or on activations that arrive quantised (x None): the
+        activation quantiser, then the int8 GEMM that decodes the resident int4 weight on the fly."""
+        N, K = self.shape
+        if int_x is None:
+            int_x = torch.empty_like(x, dtype=torch.int8)
+            scale_x = torch.empty((x.shape[0],), device=x.device, dtype=torch.float16)
+            ops.quant_fp16_to_int8(int_x, x, scale_x)
+        out = torch.empty((int_x.shape[0], N), device=int_x.device, dtype=torch.float16)
+        ops.w4a8_gemm_forward(int_x, self.qweight, self.scales_to8, self.scaled_zeros_to8, self.scales_1, scale_x, out,
+                              bias=self.bias)
+        return out
+
     @torch.no_grad()
     def _forward(self, input: torch.Tensor, batch_token_len, comp_type) -> torch.Tensor:
         N, K = self.shape
@@ -212,10 +231,12 @@ class DynamicLinear(torch.nn.Module):
         if comp_type == _W4A16_GEMV and m <= ops.GEMV_MAX_M:
             out = ops.gemv_forward(x, self.qweight, self.scales, self.scaled_zeros, m, N, K,
                                    self.group_size, bias=self.bias)
-        elif comp_type in (_W4A16_GEMM, _W4A16_GEMV):
+        elif comp_type in (_W4A16_GEMM, _W4A16_GEMV, _W4A16_ALT):
             out = ops.gemm_forward(x, self.qweight, self.scales, self.scaled_zeros, bias=self.bias)
         elif comp_type == _W8A8:
             out = self._w8a8(x, None, None)
+        elif comp_type == _W4A8:
+            out = self._w4a8(x, None, None)
         elif comp_type in (_W8A16_GEMM, _W8A16_GEMV):
             w8, _ = self._converted('i8', tiled=False)       # this lane widens int8 in registers: row-major source
             out = ops.w8a16_gemm_forward(x, w8, self.scales_1, N, bias=self.bias)

@@ -274,6 +274,36 @@ def w8a8_gemm_forward(in_feats, kernel, wscales, ascales, out_feats, bias=None, 
           ascales.data_ptr(), _ptr(bias), M, N, K, ws.data_ptr(), ws.numel(), st)
 
 
+def w4a8_gemm_forward(in_feats, qweight, scales_to8, scaled_zeros_to8, wscales, ascales, out_feats, bias=None):
+    """out_feats fp16 [M, N] <- int8 [M, K] x packed int4 [N/4, K]: the W8A8 product of the weight the int4 -> int8
+    converter would write, decoded inside the GEMM (bit-identical to dequant_interleaved_int4_to_int8 +
+    w8a8_gemm_forward; takes the place of the version-2 candidate, kairos/dynamic_linear_v2.py:161-179)."""
+    _need(in_feats, torch.int8, "in_feats"); _need(qweight, torch.int16, "qweight"); _need(out_feats, torch.float16, "out_feats")
+    _need(scales_to8, torch.float16, "scales_to8"); _need(scaled_zeros_to8, torch.float16, "scaled_zeros_to8")
+    M, K = in_feats.shape
+    N = qweight.shape[0] * 4
+    if qweight.shape[1] != K or out_feats.shape[-1] != N:
+        raise ValueError(f"w4a8_gemm_forward: activations [{M}, {K}], weight [{N}, {qweight.shape[1]}], output {tuple(out_feats.shape)}")
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
+    _call("gemm_w4a8", M, N, K, _lib.load().kmi_gemm_w4a8, out_feats.data_ptr(), in_feats.data_ptr(), qweight.data_ptr(),
+          scales_to8.data_ptr(), scaled_zeros_to8.data_ptr(), wscales.data_ptr(), ascales.data_ptr(), _ptr(bias), M, N, K,
+          GROUP_SIZE, ws.data_ptr(), ws.numel(), st)
+
+
+def w4a8_gemm_acc_i32(in_feats, qweight, scales_to8, scaled_zeros_to8):
+    """Raw int32 accumulators [M, N] of the W4A8 product."""
+    _need(in_feats, torch.int8, "in_feats"); _need(qweight, torch.int16, "qweight")
+    M, K = in_feats.shape
+    N = qweight.shape[0] * 4
+    acc = torch.empty((M, N), dtype=torch.int32, device=in_feats.device)
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
+    _lib.check(_lib.load().kmi_gemm_w4a8_acc_i32(acc.data_ptr(), in_feats.data_ptr(), qweight.data_ptr(), scales_to8.data_ptr(),
+                                                 scaled_zeros_to8.data_ptr(), M, N, K, GROUP_SIZE, ws.data_ptr(), ws.numel(), st))
+    return acc
+
+
 def w8a8_gemm_acc_i32(in_feats, kernel, N):
     """Raw int32 accumulators [M, N] of the W8A8 product."""
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel")
@@ -316,6 +346,12 @@ def f16_gemm_forward(x, w16, N, bias=None, tiled=False):
 def gemm_tile_for(M, N, K=4096):
     """Workgroup tile (64/128/256) the automatic choice uses for an M x N output over int8 rows of K bytes."""
     return _lib.load().kmi_gemm_pick_tile(int(M), int(N), int(K))
+
+
+def gemm_w4a8_tile_for(M, N, K=4096):
+    """Tile selector of the W4A8 GEMM for an M x N x K product: 128 (128 x 128), 192 (256 x 128), 256 (256 x 256) or 448
+    (256 x 256 in whole rounds, the remaining columns as 256 x 128 tiles in a second launch)."""
+    return _lib.load().kmi_gemm_w4a8_pick_tile(int(M), int(N), int(K))
 
 
 def gemm_w4a16_wp_rows(M, N, K=4096):

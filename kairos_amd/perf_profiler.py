@@ -68,6 +68,7 @@ def load_json(load_path):
 class Profiler:
     comp_type_name = COMP_TYPE_NAME
     linear_cls = DynamicLinear
+    comp_types = DEFAULT_COMP_TYPES          # candidate lanes profiling() times
 
     @torch.no_grad()
     def __init__(self, shape_list) -> None:
@@ -80,6 +81,7 @@ class Profiler:
 
     def profiling(self, **kwargs):
         for shape in self.shape_list:
+            kwargs.setdefault("comp_type_list", self.comp_types)
             seg = test_perf(str(shape), shape[1], shape[0], False, linear_cls=self.linear_cls,
                             comp_type_name=self.comp_type_name, **kwargs)
             for t in seg:
@@ -194,10 +196,15 @@ def main(argv=None):
     ap.add_argument("--n", type=int, default=200)
     ap.add_argument("--preheat", type=int, default=20)
     ap.add_argument("--max-m", type=int, default=30720)
+    ap.add_argument("--v2", action="store_true", help="version-2 id table and candidates (adds the W4A8 lane, id 7)")
     args = ap.parse_args(argv)
     # the reference's grid plus the powers of two and the half-way points of the region where the lanes cross
     grid = sorted(set([m for m in DEFAULT_INPUT_LEN if m <= args.max_m] + [1 << i for i in range(13)] + [96, 192, 384, 768, 1536]))
-    prof = Profiler(PRESETS[args.preset])
+    if args.v2:
+        from .perf_profiler_v2 import Profiler as ProfilerCls
+    else:
+        ProfilerCls = Profiler
+    prof = ProfilerCls(PRESETS[args.preset])
     details = []
     prof.profiling(input_len=grid, n=args.n, preheat_time=args.preheat, details=details)
     out = args.out if args.out.endswith("/") else args.out + "/"

@@ -25,6 +25,10 @@ Pinning status (what, other than this file agreeing with itself, fixes each func
                                   accumulated matmul, tolerance 1e-2 max-abs-rel.
   gemm_w8a16                      parity unpinned: the reference declares the id but has no
                                   implementation (kairos/dynamic_linear.py:8-9).
+  switched_forward, id 7          parity unpinned by the reference: its `w4a8_qserve` candidate calls an un-vendored
+                                  third-party GEMM with a quantiser of its own (kairos/dynamic_linear_v2.py:161-179).
+                                  The build's W4A8 lane is DEFINED as the W8A8 lane's product (same int8 weight,
+                                  decoded inside the GEMM), so its oracle is the pinned W8A8 chain, bit for bit.
   pack_int_w4a8 / trans_layout_   the reference states the layout twice (test/test_trans_layout.py:8-14 in one
   c16_to_c8                       permutation, thirdparty/Qserve/w4a8_linear.py:187-205 in two) and its own test
                                   demands trans(pack_awq(A)) == pack_w4a8(A) bit for bit (test_trans_layout.py:46-52);
@@ -434,9 +438,9 @@ def gemm_w8a16(x, w8, scales_1):
 def switched_forward(x, prep, comp_type, bias=None):
     """kairos/dynamic_linear.py:133-172 (_forward): x fp16 [M, K] -> fp16 [M, N] for one comp id."""
     name = {v: k for k, v in COMP_TYPE_NAME.items()}[comp_type]
-    if name in ("w4a16_gemv", "w4a16_gemm", "fp16"):
+    if name in ("w4a16_gemv", "w4a16_gemm", "fp16", "w4a16_marlin"):
         out = gemm_w4a16(x, prep["qweight"], prep["scales"], prep["scaled_zeros"])
-    elif name == "w8a8":
+    elif name in ("w8a8", "w4a8_qserve"):      # id 7: the build's W4A8 lane, defined as the W8A8 product without a copy
         w8 = dequant_to_i8(prep["qweight"], prep["scales_to8"], prep["scaled_zeros_to8"])
         a8, sx = quant_act_i8(x)
         out = gemm_w8a8(a8, w8, prep["scales_1"], sx)[1]

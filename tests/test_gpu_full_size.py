@@ -273,3 +273,48 @@ def test_conversion_qwen_shapes_against_oracle(ops, N, K):
     sx = torch.empty((5,), dtype=torch.float16, device="cuda")
     ops.prep_w8a8(w8, p["qweight"], p["scales_to8"], p["scaled_zeros_to8"], a8, x, sx, 128, tiled=True)
     assert np.array_equal(ops.untile(w8, N, K).cpu().numpy(), want8)
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 28672, 4096), (2048, 4096, 14336), (1024, 6144, 4096), (512, 28672, 4096),
+                                   (256, 4096, 4096), (2048, 28672, 4096), (4096, 6144, 4096)])   # the last two: two launches
+def test_w4a8_lane_full_size(ops, M, N, K):
+    """The W4A8 lane at the benchmark's sizes.  (a) On the exactly computable inputs of the W8A8 full-size test (tables
+    s = 1, z = -8, sparse +-127 activations, channel scale 1/128) the whole fp16 output is one known rounding of an
+    exact number.  (b) On the benchmark's own data (prepared N(0, 0.02) weights, outlier activations) the output equals
+    the W8A8 lane's (converter + int8 GEMM on tiled weights) bit for bit, and sampled rows equal the oracle's."""
+    rng = np.random.default_rng(N + K + M)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    w8 = q.astype(np.int8) - 8
+    Gp = O.padded_groups(K)
+    ones = torch.ones((Gp, N), dtype=torch.float16, device="cuda")
+    a = np.zeros((M, K), dtype=np.int8)
+    idx = (rng.integers(0, K, size=(M, 1)) + rng.integers(1, K // 16, size=(M, 1)) * np.arange(16)[None, :]) % K
+    np.put_along_axis(a, idx, rng.choice(np.array([-127, 127], dtype=np.int8), size=(M, 16)), axis=1)
+    sx = torch.ones((M,), dtype=torch.float16, device="cuda")
+    ws = torch.full((N,), 1.0 / 128.0, dtype=torch.float16, device="cuda")
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.w4a8_gemm_forward(dev(a), dev(O.pack_int_awq(q)), ones, ones * -8.0, ws, sx, out)
+    torch.cuda.synchronize()
+    exact = ((a.astype(np.float32) / np.float32(127.0)) @ w8.astype(np.float32).T) * np.float32(127.0 / 128.0)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), exact.astype(np.float16).view(np.uint16))
+    # (b) benchmark data
+    p = ops.prepare_weight(dev(O.synth_weights(N, K, seed=10)))
+    x_np = O.synth_acts(M, K, seed=11)
+    x = dev(x_np)
+    a8 = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    sxx = torch.empty((M,), dtype=torch.float16, device="cuda")
+    w8_t = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.prep_w8a8(w8_t, p["qweight"], p["scales_to8"], p["scaled_zeros_to8"], a8, x, sxx, 128, tiled=True)
+    want = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.w8a8_gemm_forward(a8, w8_t, p["scales_1"], sxx, want, tiled=True)
+    got = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.w4a8_gemm_forward(a8, p["qweight"], p["scales_to8"], p["scaled_zeros_to8"], p["scales_1"], sxx, got)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    rows = sample_rows(M, 4, N)
+    cols = slice(0, 512)
+    hp = {k: v.cpu().numpy() for k, v in p.items()}
+    w8_ref = O.dequant_to_i8(hp["qweight"][: 512 // 4], hp["scales_to8"][:, cols], hp["scaled_zeros_to8"][:, cols])
+    a8_ref, sx_ref = O.quant_act_i8(x_np[rows])
+    ref = O.gemm_w8a8(a8_ref, w8_ref, hp["scales_1"][cols], sx_ref)[1]
+    assert np.array_equal(got[torch.from_numpy(rows).cuda()][:, cols].cpu().numpy().view(np.uint16), ref.view(np.uint16))

@@ -266,6 +266,65 @@ def test_gemm_w8a8_path(ops, M, tile):
     assert_same_bits(host(out), ref)
 
 
+@pytest.mark.parametrize("tile", [0, 128, 192, 256])
+@pytest.mark.parametrize("M", GEMM_M)
+def test_gemm_w4a8_bit_exact(ops, M, tile):
+    """W4A8 (int4 weights decoded to the converter's int8 values inside the int8 MFMA GEMM): int32 accumulators and
+    fp16 outputs against the oracle's W8A8 chain, bit for bit; N = 384 leaves both tiles ragged."""
+    N, K = 384, 1024
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=700 + M)
+    a8, sx = O.quant_act_i8(x)
+    acc_ref, out_ref = O.gemm_w8a8(a8, p["w8"], p["scales_1"], sx)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float16)
+    out_b_ref = (out_ref.astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    qw, s8, z8 = dev(p["qweight"]), dev(p["scales_to8"]), dev(p["scaled_zeros_to8"])
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    out_b = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(1)
+    try:
+        acc = ops.w4a8_gemm_acc_i32(dev(a8), qw, s8, z8)
+        ops.w4a8_gemm_forward(dev(a8), qw, s8, z8, dev(p["scales_1"]), dev(sx), out)
+        ops.w4a8_gemm_forward(dev(a8), qw, s8, z8, dev(p["scales_1"]), dev(sx), out_b, bias=dev(bias))
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert_same_bits(host(acc), acc_ref)
+    assert_same_bits(host(out), out_ref)
+    assert_same_bits(host(out_b), out_b_ref)
+
+
+@pytest.mark.parametrize("tile,splits", [(128, 1), (256, 1), (128, 3), (256, 2), (192, 1), (192, 4), (0, 0)])
+def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
+    """Arbitrary tables (every table byte differs from row to row and group to group, values beyond the int8 range are
+    clipped as the converter clips them), full-range activations, K split over workgroups: accumulators equal the
+    oracle's and the W8A8 GEMM's on the converter's output."""
+    rng = np.random.default_rng(tile + splits)
+    N, K, M = 512, 2048, 200
+    Gp = O.padded_groups(K)
+    qw_np = rng.integers(-32768, 32768, size=(N // 4, K), dtype=np.int16)
+    s_np = (rng.random((Gp, N), dtype=np.float32) * 17.5 + 0.01).astype(np.float16)
+    z_np = (rng.standard_normal((Gp, N), dtype=np.float32) * 70.0).astype(np.float16)
+    a8_np = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w8_ref = O.dequant_to_i8(qw_np, s_np, z_np)
+    assert w8_ref.min() == -128 and w8_ref.max() == 127           # the clip is exercised
+    qw, s8, z8, a8 = dev(qw_np), dev(s_np), dev(z_np), dev(a8_np)
+    w8 = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(w8, qw, s8, z8, 128)
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(splits)
+    try:
+        acc = ops.w4a8_gemm_acc_i32(a8, qw, s8, z8)
+        again = ops.w4a8_gemm_acc_i32(a8, qw, s8, z8)
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert_same_bits(host(w8), w8_ref)
+    assert_same_bits(host(acc), O.gemm_i8_acc(a8_np, w8_ref))
+    assert torch.equal(acc, again) and torch.equal(acc, ops.w8a8_gemm_acc_i32(a8, w8, N))
+
+
 @pytest.mark.parametrize("tile", [64, 128, 256])
 @pytest.mark.parametrize("M", GEMM_M)
 def test_gemm_w4a16_f16_w8a16(ops, M, tile):
