@@ -141,15 +141,23 @@ int kmi_trans_layout_w4a8(void* out_i8, const void* qweight, int N, int K, void*
 /* out = x . dequant(qweight)^T (+bias), weights streamed once, fp32 accumulation on MFMA.
  * Replaces gemv_forward_cuda_new (thirdparty/AWQ/kernels/csrc/pybind.cpp:23,
  * thirdparty/AWQ/kernels/csrc/quantization_new/gemv/gemv_cuda.cu:245-463).
- * Needs 1<=M<=KMI_GEMV_MAX_M, G==128, N%16==0, K%128==0. */
+ * Needs 1<=M<=KMI_GEMV_MAX_M, G==128, N%16==0, K%128==0.
+ * workspace (optional, NULL = none): caller-owned device scratch that lets long, narrow weights split K over
+ * several workgroups per column strip.  Layout: the first KMI_GEMV_WS_HEADER bytes hold arrival counters, which must be
+ * ZERO before the first call that uses the buffer and are zero again when every call's kernel has finished; fp32 partial
+ * sums follow.  Calls that share a workspace must be ordered on one stream.  Results do not depend on which
+ * workgroup finishes last (partial sums are added in split order); the split count depends on the arguments only. */
+#define KMI_GEMV_WS_HEADER 65536
 int kmi_gemv_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
-                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
+                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
-/* Tuning variant: nt = 16-column tiles per wave (1,2,4), nw = waves per workgroup (4,8,16);
- * nt<=0 or nw<=0 selects the built-in heuristic.  No reference counterpart. */
+/* Tuning variant: nt = 16-column tiles per wave (1..8), nw = waves per workgroup (4,8,16), ks = workgroups that share
+ * the K range of one column strip (1 = no split; more needs a workspace of KMI_GEMV_WS_HEADER + ks*M*N*4 bytes);
+ * nt<=0 or nw<=0 selects the built-in heuristic for all three.  No reference counterpart. */
 int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
                        const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
-                       int nt, int nw, void* stream);
+                       int nt, int nw, int ks, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- MFMA GEMMs, any M -------------------------------------------------------------------------
  *

@@ -29,8 +29,8 @@ SIGNATURES = {
     "kmi_prepare_weight": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "kmi_padded_groups": [_I, _I],
     "kmi_trans_layout_w4a8": [_P, _P, _I, _I, _P],
-    "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _Z, _P],
     # GEMMs end with (workspace pointer, workspace bytes, stream)
     "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w4a16_noalloc": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

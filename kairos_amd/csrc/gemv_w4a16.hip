@@ -15,6 +15,14 @@
 // four-row interleave makes a 16-row strip one contiguous K*8-byte region.  Partial sums meet in
 // LDS and are added in a fixed order (deterministic output).
 //
+// Long, narrow weights (K much larger than N: 4096 x 14336, 8192 x 28672) have too few column strips to keep enough
+// loads in flight and make every workgroup read the whole activation matrix.  There K is also split over KS
+// workgroups per column strip (grid.y): each writes its fp32 partial sums to caller-owned scratch and bumps a per-strip
+// counter; whichever workgroup arrives last adds the KS partial sums in split order (deterministic), applies bias and
+// writes the output.  Nobody ever waits for another workgroup.  Partial sums and the counter travel through
+// agent-scope atomic stores, loads and one atomic add (coherent across the XCDs' L2 caches without cache
+// write-backs); a thread waits for its own stores to complete before the workgroup's arrival is counted.
+//
 // Lane roles inside a wave, for one K group and one 16-column tile: lane = (r16, j), r16 = lane&15,
 // j = lane>>4.  The lane loads the 16-byte chunk of row n = tile*16 + r16 that covers
 // k = 128c + 32j .. +31; nibble plane a of its four words holds the eight K-contiguous weights
@@ -28,7 +36,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
                                                              const u4_t* __restrict__ qw,
                                                              const half_t* __restrict__ scales,
                                                              const half_t* __restrict__ szeros,
-                                                             const half_t* __restrict__ bias, int M, int N, int K) {
+                                                             const half_t* __restrict__ bias, int M, int N, int K,
+                                                             float* __restrict__ partial, uint32_t* __restrict__ counters) {
     extern __shared__ float red[];               // [NW][MT*NT*4][64]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -40,7 +49,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
     const int nblk = gridDim.x, xcd = blockIdx.x & 7;
     const int strip = xcd * (nblk >> 3) + min(xcd, nblk & 7) + (blockIdx.x >> 3);
     const int n0 = strip * (16 * NT);
-    const int ngroups = K >> 7;
+    const int KS = gridDim.y, ks = blockIdx.y;              // K split over workgroups: this one covers groups [g0, g1)
+    const int all_groups = K >> 7;
+    const int g0 = (int)((long)ks * all_groups / KS), ngroups = (int)((long)(ks + 1) * all_groups / KS);
     const int kq = K >> 3;                       // 16-byte units per fp16 row of x / per four-row weight block
 
     f4_t acc[MT][NT];
@@ -76,7 +87,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
     constexpr int U = (MT == 1 && NT <= 2) ? 2 : 1;
     const h8_t ones = {(half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1};
     const h8_t sixteenth = ones * (half_t)0.0625f;
-    for (int c0 = wave; c0 < ngroups; c0 += NW * U) {
+    for (int c0 = g0 + wave; c0 < ngroups; c0 += NW * U) {
         u4_t u[U][NT];
         half_t sz[U][NT];
         h8_t xa[U][MT][4];
@@ -155,6 +166,25 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
             for (int i = 0; i < 4; ++i) red[(wave * R + (mt * NT + nt) * 4 + i) * 64 + lane] = acc[mt][nt][i];
     __syncthreads();
 
+    if (KS == 1) {
+        for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
+            const int l = idx & 63, reg = idx >> 6;
+            const int i = reg & 3, t = reg >> 2;
+            const int nt = t % NT, mt = t / NT;
+            const int m = mt * 16 + 4 * (l >> 4) + i;
+            const int n = n0 + nt * 16 + (l & 15);
+            if (m < M && n < N) {
+                half_t h = (half_t)v;
+                if (bias) h = (half_t)((float)h + (float)bias[n]);
+                out[(long)m * N + n] = h;
+            }
+        }
+        return;
+    }
+    // ---- K split over workgroups: publish this workgroup's partial sums, count the arrival, last one finishes
     for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
         float v = 0.f;
 #pragma unroll
@@ -164,15 +194,34 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
         const int nt = t % NT, mt = t / NT;
         const int m = mt * 16 + 4 * (l >> 4) + i;
         const int n = n0 + nt * 16 + (l & 15);
+        if (m < M && n < N)
+            __hip_atomic_store(partial + ((long)ks * M + m) * N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this thread's partial sums have been performed
+    __shared__ uint32_t arrived;
+    __syncthreads();                                         // ... and everybody else's in the workgroup
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counters + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrived != (uint32_t)(KS - 1)) return;               // workgroup-uniform
+    for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
+        const int l = idx & 63, reg = idx >> 6;
+        const int i = reg & 3, t = reg >> 2;
+        const int nt = t % NT, mt = t / NT;
+        const int m = mt * 16 + 4 * (l >> 4) + i;
+        const int n = n0 + nt * 16 + (l & 15);
         if (m < M && n < N) {
+            float v = 0.f;
+            for (int q = 0; q < KS; ++q)                     // split order: the same sum whoever arrives last
+                v += __hip_atomic_load(partial + ((long)q * M + m) * N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             half_t h = (half_t)v;
             if (bias) h = (half_t)((float)h + (float)bias[n]);
             out[(long)m * N + n] = h;
         }
     }
+    if (threadIdx.x == 0) __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
-typedef void (*gemv_fn)(half_t*, const half_t*, const u4_t*, const half_t*, const half_t*, const half_t*, int, int, int);
+typedef void (*gemv_fn)(half_t*, const half_t*, const u4_t*, const half_t*, const half_t*, const half_t*, int, int, int, float*, uint32_t*);
 
 template <int MT, int NT, int NW>
 static constexpr bool gemv_cfg_ok() {
@@ -231,7 +280,7 @@ static gemv_fn gemv_lookup(int mt, int nt, int nw) {
 //   Waves per workgroup over K (nw): eight; sixteen for a single column tile at the smallest M, where the kernel is
 //   a pure latency chain (4096 x 14336 at M=1: 10.4 against 11.9 us); four from three row tiles on (M > 32), and for
 //   seven or eight column tiles when more than one workgroup shares a CU (57344 x 8192 at M=16: 45.3 against 48.5 us).
-static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_out) {
+static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_out, int* ks_out) {
     const int strips = (N + 15) / 16, groups = K / 128;
     const double c = M <= 4 ? 0.6 : M <= 8 ? 1.0 : M <= 16 ? 1.7 : 2.5;
     int nt = 1, wgs = strips;
@@ -253,35 +302,69 @@ static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_o
     while (nw > 4 && (groups < nw || gemv_lookup(mt, nt, nw) == nullptr)) nw >>= 1;
     *nt_out = nt;
     *nw_out = nw;
+    *ks_out = 1;
+    // Long, narrow weights: few column strips, each a long walk over K.  A wave then runs several load-wait-compute
+    // trips in a row and every workgroup reads the whole activation matrix.  Split K over ks workgroups per strip
+    // so that strips / nt * ks stays near 256, with wider column tiles as M grows.  Measured (us, before -> after):
+    // 4096 x 14336  M=1 10.8 -> 9.5, M=8 13.6 -> 10.6, M=16 16.7 -> 12.0, M=32 29.0 -> 17.4;  8192 x 28672  M=16
+    // 36.3 -> 29.1, M=32 58.2 -> 42.5;  4096 x 4096  M=32 10.2 -> 9.4;  8192 x 8192  M=32 18.7 -> 17.1.  Short rows
+    // (K = 4096 at M <= 16, K = 8192 at M <= 16) lose to the unsplit kernel and keep it.
+    if (mt <= 2 && strips <= 512 && ((mt == 1 && groups >= 96) || (mt == 2 && groups >= 32))) {
+        int want_nt = M <= 4 ? 2 : M <= 8 ? (strips > 256 ? 4 : 2) : (mt == 2 && groups < 64) ? 2 : 4;
+        while (want_nt > 1 && gemv_lookup(mt, want_nt, 8) == nullptr) want_nt >>= 1;
+        int ks = (256 * want_nt + strips / 2) / strips;
+        if (ks > 8) ks = 8;
+        int want_nw = (M <= 4 && gemv_lookup(mt, want_nt, 16) != nullptr) ? 16 : 8;
+        while (ks > 1 && groups / ks < want_nw) --ks;
+        if (ks >= 2) {
+            *nt_out = want_nt;
+            *nw_out = want_nw;
+            *ks_out = ks;
+        }
+    }
 }
 
 extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
                                   const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
-                                  int nt, int nw, void* stream) {
+                                  int nt, int nw, int ks, void* workspace, size_t workspace_bytes, void* stream) {
     if (!out_f16 || !x_f16 || !qweight || !scales || !scaled_zeros)
         return kmi_set_error(KMI_E_NULL, "kmi_gemv_w4a16: NULL pointer argument");
-    if (!kmi_aligned16(x_f16) || !kmi_aligned16(qweight))
-        return kmi_set_error(KMI_E_ALIGN, "kmi_gemv_w4a16: x and qweight must be 16-byte aligned");
+    if (!kmi_aligned16(x_f16) || !kmi_aligned16(qweight) || (workspace && !kmi_aligned16(workspace)))
+        return kmi_set_error(KMI_E_ALIGN, "kmi_gemv_w4a16: x, qweight and workspace must be 16-byte aligned");
     if (G != 128) return kmi_set_error(KMI_E_GROUP, "kmi_gemv_w4a16: group size %d unsupported (128 only)", G);
     if (M < 1 || M > KMI_GEMV_MAX_M)
         return kmi_set_error(KMI_E_M_RANGE, "kmi_gemv_w4a16: M=%d outside 1..%d", M, KMI_GEMV_MAX_M);
     if (N <= 0 || K <= 0 || (N & 15) || (K & 127))
         return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: need N%%16==0 and K%%128==0, got N=%d K=%d", N, K);
     const int mt = (M + 15) / 16;
-    if (nt <= 0 || nw <= 0) gemv_default_cfg(M, mt, N, K, &nt, &nw);
+    const bool automatic = nt <= 0 || nw <= 0;
+    if (automatic) gemv_default_cfg(M, mt, N, K, &nt, &nw, &ks);
+    if (ks < 1) ks = 1;
     gemv_fn fn = gemv_lookup(mt, nt, nw);
     if (!fn) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: no kernel for m-tiles=%d nt=%d nw=%d", mt, nt, nw);
-    const int strips = N / 16;
-    const dim3 grid((strips + nt - 1) / nt), block(nw * 64);
+    const int strips = N / 16, wg_x = (strips + nt - 1) / nt, groups = K / 128;
+    // a split over K needs scratch: [KMI_GEMV_WS_HEADER bytes of per-strip arrival counters, zero between calls]
+    // [ks x M x N fp32 partial sums]; without it (or with too little) the call runs unsplit
+    if (ks > groups) ks = groups;
+    const size_t need = (size_t)KMI_GEMV_WS_HEADER + (size_t)ks * M * N * sizeof(float);
+    if (ks > 1 && (workspace == nullptr || workspace_bytes < need || (size_t)wg_x * sizeof(uint32_t) > KMI_GEMV_WS_HEADER)) {
+        if (!automatic) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: %d K splits need %zu bytes of workspace", ks, need);
+        ks = 1;
+    }
+    const dim3 grid(wg_x, ks), block(nw * 64);
     const size_t lds = (size_t)nw * mt * nt * 4 * 64 * sizeof(float);
+    uint32_t* counters = static_cast<uint32_t*>(workspace);
+    float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + KMI_GEMV_WS_HEADER) : nullptr;
     hipLaunchKernelGGL(fn, grid, block, lds, static_cast<hipStream_t>(stream), static_cast<half_t*>(out_f16),
                        static_cast<const half_t*>(x_f16), static_cast<const u4_t*>(qweight),
                        static_cast<const half_t*>(scales), static_cast<const half_t*>(scaled_zeros),
-                       static_cast<const half_t*>(bias), M, N, K);
+                       static_cast<const half_t*>(bias), M, N, K, partial, counters);
     return kmi_check_launch("kmi_gemv_w4a16");
 }
 
 extern "C" int kmi_gemv_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
-                              const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream) {
-    return kmi_gemv_w4a16_cfg(out_f16, x_f16, qweight, scales, scaled_zeros, bias, M, N, K, G, 0, 0, stream);
+                              const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+    return kmi_gemv_w4a16_cfg(out_f16, x_f16, qweight, scales, scaled_zeros, bias, M, N, K, G, 0, 0, 0, workspace,
+                              workspace_bytes, stream);
 }

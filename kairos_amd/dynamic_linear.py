@@ -175,8 +175,12 @@ class DynamicLinear(torch.nn.Module):
                                         ops._lib.load().kmi_gemv_w4a16, input.device.index or 0)
         N, K = self.shape
         out = torch.empty(shape[:-1] + (N,), dtype=torch.float16, device=input.device)
+        st = ops._raw_stream(ptrs[5]) if ops._raw_stream is not None else ops._stream()
+        ws = ops._gemv_workspaces.get((ptrs[5], st))
+        if ws is None:
+            ws = ops.gemv_workspace_for(input.device, st)
         rc = ptrs[4](out.data_ptr(), input.data_ptr(), ptrs[0], ptrs[1], ptrs[2], ptrs[3], m, N, K, self.group_size,
-                     ops._raw_stream(ptrs[5]) if ops._raw_stream is not None else ops._stream())
+                     ws.data_ptr(), ws.numel(), st)
         if rc < 0:
             ops._lib.check(rc)
         return out

@@ -203,13 +203,17 @@ def _flat2d(x):
 
 
 def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZE, bias=None, cfg=None):
-    """W4A16 for small m (gemv_cuda.cu:245-463).  Returns fp16 [*x.shape[:-1], n]."""
+    """W4A16 for small m (gemv_cuda.cu:245-463).  Returns fp16 [*x.shape[:-1], n].  cfg: (column tiles per wave, waves
+    per workgroup[, workgroups over K]) for tuning; None = the library's choice."""
     _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
     out = torch.empty(x.shape[:-1] + (n,), dtype=torch.float16, device=x.device)
     lib = _lib.load()
-    nt, nw = cfg if cfg is not None else (0, 0)
+    nt, nw, ks = (tuple(cfg) + (1,))[:3] if cfg is not None else (0, 0, 0)
+    st = _stream()
+    ws = gemv_workspace_for(x.device, st)
     _call("gemv_w4a16", m, n, k, lib.kmi_gemv_w4a16_cfg, out.data_ptr(), x.data_ptr(), qweight.data_ptr(),
-          scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, _stream())
+          scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, ks, ws.data_ptr(),
+          ws.numel(), st)
     return out
 
 
@@ -232,14 +236,34 @@ def workspace_for(device, stream=None):
     return ws
 
 
+GEMV_WORKSPACE_BYTES = 65536 + (32 << 20)      # arrival counters (KMI_GEMV_WS_HEADER) + fp32 partial sums
+_gemv_workspaces = {}
+
+
+def gemv_workspace_for(device, stream=None):
+    """Scratch of the small-M kernel's split over K, per (device, stream) like workspace_for, but ZEROED at creation:
+    its first 64 KiB are arrival counters that the kernels return to zero themselves.  Kept apart from the GEMM
+    scratch, whose partial sums would overwrite the counters."""
+    dev = torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if stream is None:
+        stream = _stream()
+    ws = _gemv_workspaces.get((idx, stream))
+    if ws is None:
+        ws = _gemv_workspaces[(idx, stream)] = torch.zeros(GEMV_WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+    return ws
+
+
 def ensure_workspace(device="cuda", stream=None):
     """Creates the calling (or given) stream's split-K scratch ahead of time, e.g. before a graph capture on it."""
+    gemv_workspace_for(device, stream)
     return workspace_for(device, stream)
 
 
 def drop_workspaces():
     """Forgets every scratch buffer (tests).  Not while a captured graph that used one is still alive."""
     _workspaces.clear()
+    _gemv_workspaces.clear()
 
 
 def gemm_splits_for(lane, M, N, K, workspace_bytes=WORKSPACE_BYTES):

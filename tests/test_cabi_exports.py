@@ -41,9 +41,10 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_cvt_i4_to_i8(16, 16, 16, 16, 4, 128, 64, None) == -3
     assert lib.kmi_cvt_i4_to_i8(16, 16, 16, 16, 6, 128, 128, None) == -2
     assert lib.kmi_cvt_i4_to_i8(16, 8, 16, 16, 4, 128, 128, None) == -5
-    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 0, 64, 128, 128, None) == -4
-    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 65, 64, 128, 128, None) == -4
-    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 4, 60, 128, 128, None) == -2
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 0, 64, 128, 128, None, 0, None) == -4
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 65, 64, 128, 128, None, 0, None) == -4
+    assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 4, 60, 128, 128, None, 0, None) == -2
+    assert lib.kmi_gemv_w4a16_cfg(16, 16, 16, 16, 16, None, 4, 64, 1024, 128, 1, 8, 2, None, 0, None) == -2   # a forced K split needs scratch
     assert lib.kmi_gemm_w8a8(16, 16, 16, 16, 16, None, 4, 64, 100, None, 0, None) == -2
     assert lib.kmi_gemm_w8a8(16, 16, 16, None, 16, None, 4, 64, 128, None, 0, None) == -1
     assert lib.kmi_quant_act_i8(16, 16, 16, 4, 12, None) == -2

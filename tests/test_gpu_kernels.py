@@ -204,6 +204,27 @@ def test_gemv_default_split_on_unbalanced_widths(ops, N):
         assert O.max_abs_rel(host(out), O.gemm_f16(x, p["w16"])) < 2e-3
 
 
+@pytest.mark.parametrize("M,nt,nw,ks", [(1, 1, 16, 2), (3, 2, 8, 4), (8, 4, 8, 7), (16, 4, 8, 8), (20, 2, 8, 3), (40, 2, 4, 2), (64, 1, 8, 4)])
+def test_gemv_split_over_workgroups(ops, M, nt, nw, ks):
+    """K split over several workgroups per column strip (long, narrow weights): the workgroup that arrives last adds the
+    partial sums in split order, so the result is the same on every call; the arrival counters are zero again afterwards
+    and a second call on the same scratch works; bias applied once."""
+    N, K = 320, 3584                                         # 28 groups: uneven over 3, 7 and 8 splits; ragged last strip
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=40 + M)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float16)
+    ref = (O.gemm_w4a16(x, p["qweight"], p["scales"], p["scaled_zeros"]).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    args = (dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+    outs = [ops.gemv_forward(*args, bias=dev(bias), cfg=(nt, nw, ks)) for _ in range(4)]
+    torch.cuda.synchronize()
+    assert O.max_abs_rel(host(outs[0]), ref) < 2e-3
+    assert all(torch.equal(outs[0].view(torch.int16), o.view(torch.int16)) for o in outs[1:])
+    ws = ops.gemv_workspace_for("cuda")
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
+    unsplit = ops.gemv_forward(*args, bias=dev(bias), cfg=(nt, nw, 1))
+    assert O.max_abs_rel(host(outs[0]), host(unsplit)) < 1e-3
+
+
 def test_gemv_bias_and_ragged_strip(ops):
     N, K, M = 48, 256, 4                                    # N is not a multiple of the 64-column strip
     p = prep(N, K)
