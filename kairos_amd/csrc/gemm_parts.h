@@ -234,7 +234,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
 #pragma unroll
                 for (int k = 0; k < NK; ++k) {
                     const int m = mw + i * 32 + (k * 64 + lane) / CPR;
+#ifdef KMI_TEST_EPI_PLAIN
+                    if (m < M && n < N) *reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N) = v[k];
+#else
                     if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N));
+#endif
                 }
             } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
 #pragma unroll
@@ -275,7 +279,11 @@ __device__ __forceinline__ void sched_interleave() {
 // in column-major groups of GROUP_M tile rows, so the tiles resident on one XCD at a time form a
 // compact block that shares A row-panels and B column-panels in that XCD's L2.
 __device__ __forceinline__ void tile_of_block(int wg, int TM, int TN, int& tm, int& tn) {
+#ifdef KMI_TEST_GROUP_M
+    constexpr int XCDS = 8, GROUP_M = KMI_TEST_GROUP_M;
+#else
     constexpr int XCDS = 8, GROUP_M = 8;
+#endif
     const int total = TM * TN;
     const int xcd = wg % XCDS, q = wg / XCDS;
     const int base = total / XCDS, rem = total % XCDS;

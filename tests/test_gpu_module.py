@@ -387,3 +387,52 @@ def test_decoder_harness_two_layers(gpu):
             ref.free()
     finally:
         DynamicLinear.prof = old
+
+
+def test_smooth_scale_search_with_the_library_probe(gpu):
+    """The smoothing-scale search (kairos/smooth_scale.py:66-176) with its default probe -- the library's own quantised
+    linear through the W4A8 lane -- on a tiny fp16 Llama with outlier channels: the scales it finds lower the error of
+    the quantised model (every linear a DynamicLinear on the int8-activation lane) against the fp16 model."""
+    transformers = pytest.importorskip("transformers")
+    from kairos.dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear
+    from kairos.perf_profiler_v2 import Profiler
+    from kairos.quant_model import get_name_linears, quantize_model
+    from kairos.smooth_scale import apply_scale, smooth_scale
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=128, max_position_embeddings=256)
+    model = transformers.LlamaForCausalLM(cfg).half().cuda().eval()
+    with torch.no_grad():
+        for layer in model.model.layers:
+            layer.input_layernorm.weight[::37] *= 30.0
+            layer.post_attention_layernorm.weight[::41] *= 30.0
+    ids = torch.randint(0, 128, (2, 48), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    with torch.no_grad():
+        want = model(ids).logits.float()
+    meta = smooth_scale(model, {"input_ids": ids})
+    assert len(meta) == 2 and all(len(b) == 3 for b in meta)
+    assert all(type(m) is torch.nn.Linear for layer in model.model.layers for m in get_name_linears(layer).values())
+    with torch.no_grad():
+        assert torch.equal(model(ids).logits.float(), want)                      # the search left the model as it was
+
+    shapes = sorted({tuple(m.weight.shape) for layer in model.model.layers for m in get_name_linears(layer).values()})
+    prof = Profiler(shapes)
+    for s in shapes:
+        prof.record_best_comp(s, 1 << 20, 'w4a8_qserve')
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+
+    def quantised_error(smoothed):
+        m = transformers.LlamaForCausalLM(cfg).half().cuda().eval()
+        m.load_state_dict(model.state_dict())
+        if smoothed:
+            apply_scale(m, meta)
+        quantize_model(m, quant_strategy='DynamicLinear', version='2')
+        with torch.no_grad():
+            return (m(ids).logits.float() - want).pow(2).mean().item()
+
+    try:
+        plain, smoothed = quantised_error(False), quantised_error(True)
+    finally:
+        DynamicLinear.prof = old
+    assert smoothed < plain, (plain, smoothed)

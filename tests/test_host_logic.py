@@ -360,6 +360,57 @@ def test_apply_scale_keeps_the_fp_function():
         apply_scale(model, [[("no_such_op", ["mlp.down_proj"], torch.ones(1, 512))]])
 
 
+def test_smooth_scale_search_finds_scales_that_help():
+    """kairos/smooth_scale.py:66-176 with the plain-torch probe (no GPU): on a tiny Llama whose norm weights give a few
+    channels 30x the magnitude of the rest, the search returns one entry per block in the reference's format, prefers a
+    non-trivial exponent for the blocks behind the norms, leaves the model untouched, and folding its scales in lowers
+    the error of the quantised probes against the unquantised model."""
+    from kairos.smooth_scale import apply_scale, fake_quant_probe, smooth_scale
+    from kairos.quant_model import get_name_linears, set_op_by_name
+    model = _tiny_llama(seed=5).float()
+    with torch.no_grad():
+        for layer in model.model.layers:
+            layer.input_layernorm.weight[::37] *= 30.0
+            layer.post_attention_layernorm.weight[::41] *= 30.0
+    ids = torch.randint(0, 128, (2, 24), generator=torch.Generator().manual_seed(0))
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    with torch.no_grad():
+        want = model(ids).logits
+    meta = smooth_scale(model, {"input_ids": ids}, make_probe=fake_quant_probe)
+    assert all(torch.equal(v, state[k]) for k, v in model.state_dict().items())       # the search restores everything
+    assert all(type(m) is torch.nn.Linear for layer in model.model.layers for m in get_name_linears(layer).values())
+    assert len(meta) == 2
+    for blocks in meta:
+        assert [b[0] for b in blocks] == ["input_layernorm", "post_attention_layernorm", "mlp.up_proj"]
+        assert [b[1] for b in blocks] == [["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"],
+                                          ["mlp.gate_proj", "mlp.up_proj"], ["mlp.down_proj"]]
+        assert [tuple(b[2].shape) for b in blocks] == [(1, 256), (1, 256), (1, 512)]
+        for _prev, _names, sc in blocks:
+            assert torch.isfinite(sc).all() and (sc > 0).all()
+            assert abs(float(sc.max() * sc.min()) - 1.0) < 1e-3                        # normalised by sqrt(max * min)
+        assert float(blocks[0][2].max() / blocks[0][2].min()) > 2.0                    # outlier channels get scaled down
+
+    def quantised_error(m):
+        """logits of `m` with every decoder linear replaced by the fake-quant probe (unit scales) against `want`"""
+        originals = []
+        for layer in m.model.layers:
+            for name, lin in get_name_linears(layer).items():
+                originals.append((layer, name, lin))
+                set_op_by_name(layer, name, fake_quant_probe(lin, torch.ones(1, lin.in_features)))
+        with torch.no_grad():
+            err = (m(ids).logits - want).pow(2).mean().item()
+        for layer, name, lin in originals:
+            set_op_by_name(layer, name, lin)
+        return err
+
+    plain = quantised_error(model)
+    apply_scale(model, meta)
+    with torch.no_grad():
+        assert torch.allclose(model(ids).logits, want, rtol=1e-3, atol=1e-3)           # smoothing keeps the function
+    smoothed = quantised_error(model)
+    assert smoothed < plain, (plain, smoothed)
+
+
 def test_matched_norm_asks_its_consumers_for_their_lane():
     """Host half of activation matching: the formats a norm emits follow the table lookups of its consumers
     (int8 where a lane is W8A8, fp16 elsewhere, both when consumers disagree); no GPU involved."""
