@@ -15,6 +15,7 @@
 // W4A16 products of up to ~1000 rows run gemm_w4a16_wp_kernel instead (weights decoded in registers by the wave
 // that owns their columns, never written to LDS); the host side at the end of the file picks kernel and tile.
 #include "gemm_parts.h"
+#include <atomic>
 #include <mutex>
 
 template <int KIND, int BM, int BN, bool TILED_B>
@@ -571,7 +572,7 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
 // fetches the chunk that belongs in slot l.  The tiled weight layout ([N/128][K-stages][128][64 B],
 // already swizzled) makes the B side a straight 8 KiB copy per 128-row strip.
 
-template <int KIND, int BM, int BN, bool TILED_B, int NS>
+template <int KIND, int BM, int BN, bool TILED_B, int NS, bool PERSIST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((NS == 3 && BM == 256 && BN == 128) ? 2 : 1)))
 void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for two workgroups per CU: <= 256 registers, 72 KiB of LDS
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass cannot instantiate code that uses the buffer resource type
@@ -582,6 +583,7 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
     constexpr int STAGE = ROWS * 64;
     constexpr int NLD = ROWS * 4 / 256;                     // direct loads per thread per stage
     static_assert(BM % 64 == 0 && BN % 64 == 0 && NLD * 64 == ROWS, "each wave-load fills 16 rows");
+    static_assert(!PERSIST || NS == 4, "the persistent form keeps two stages of the next tile beside the epilogue's patches");
     using acc_t = typename std::conditional<I8, i16_t, f16_t>::type;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -590,74 +592,77 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: feeds M0
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
-    int tm, tn;
     const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + BN - 1) / BN;
-    const int split = blockIdx.x / (TM_ * TN_);
-    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
-    const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
+    const int nvirt = TM_ * TN_ * p.splits;                  // tiles x splits: the units of work
     const long row_bytes = I8 ? (long)K : (long)K * 2;
     const int T_all = (int)(row_bytes >> 6);                // 64-byte stages along K
     const int t_per = (T_all + p.splits - 1) / p.splits;
-    const int t0 = split * t_per;                            // this workgroup covers stages t0 .. t0+T-1
-    const int T = (t0 + t_per <= T_all) ? t_per : T_all - t0;
-
-    acc_t acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     // ---- global sources.  Load i of wave w fills the KiB region R = 4*i + w = rows 16R .. 16R+15.
     // Addresses are a wave-uniform base (advanced per k-stage with scalar adds) plus a per-lane
-    // 32-bit offset that never changes, so the loop carries no vector address arithmetic.
+    // 32-bit offset that never changes within a tile, so the loop carries no vector address arithmetic.
+    // A unit of work: its place in the output, its K range and the per-lane offsets of its loads.  The
+    // persistent form folds the weight strip of the tile into the offsets (the host checks that they fit
+    // 32 bits); the one-tile form moves the base pointer instead.
+    struct Unit { int split, m0, n0, t0, T; uint32_t voff[NLD]; };
+    auto setup = [&](int vb, Unit& u) {
+        int tm, tn;
+        u.split = vb / (TM_ * TN_);
+        tile_of_block(vb - u.split * (TM_ * TN_), TM_, TN_, tm, tn);
+        u.m0 = tm * BM;
+        u.n0 = p.n_begin + tn * BN;
+        u.t0 = u.split * t_per;                              // this unit covers stages t0 .. t0+T-1
+        u.T = (u.t0 + t_per <= T_all) ? t_per : T_all - u.t0;
+        const long fold = (TILED_B && PERSIST) ? (long)(u.n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64) : 0;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int row = 16 * (4 * i + wave) + (lane >> 2);
+            const int pc = lane & 3;
+            const int c = pc ^ ((row >> 2) & 3);
+            if (16 * (4 * i) < BM) {                         // region lies in the A part (BM % 64 == 0)
+                int m = u.m0 + row;
+                m = m < M ? m : M - 1;
+                u.voff[i] = (uint32_t)((long)m * row_bytes + c * 16);
+            } else if constexpr (TILED_B) {
+                const int rb = row - BM;
+                int strip = rb >> 7;
+                if (u.n0 + strip * KMI_TILE_N >= N) strip = 0;
+                u.voff[i] = (uint32_t)(fold + (long)strip * T_all * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
+            } else {
+                int n = u.n0 + row - BM;
+                n = n < N ? n : N - 1;
+                u.voff[i] = (uint32_t)((long)n * row_bytes + c * 16);
+            }
+        }
+    };
+    Unit cur;
+    setup(blockIdx.x, cur);
+
     const char* a_base = static_cast<const char*>(p.a);
     const char* b_base = static_cast<const char*>(p.b);
-    if constexpr (TILED_B) b_base += (long)(n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64);
+    if constexpr (TILED_B && !PERSIST) b_base += (long)(cur.n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64);
     constexpr long B_STEP = TILED_B ? KMI_TILE_N * 64 : 64;
-    uint32_t voff[NLD];
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        const int row = 16 * (4 * i + wave) + (lane >> 2);
-        const int pc = lane & 3;
-        const int c = pc ^ ((row >> 2) & 3);
-        if (16 * (4 * i) < BM) {                             // region lies in the A part (BM % 64 == 0)
-            int m = m0 + row;
-            m = m < M ? m : M - 1;
-            voff[i] = (uint32_t)((long)m * row_bytes + c * 16);
-        } else if constexpr (TILED_B) {
-            const int rb = row - BM;
-            int strip = rb >> 7;
-            if (n0 + strip * KMI_TILE_N >= N) strip = 0;
-            voff[i] = (uint32_t)((long)strip * T_all * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
-        } else {
-            int n = n0 + row - BM;
-            n = n < N ? n : N - 1;
-            voff[i] = (uint32_t)((long)n * row_bytes + c * 16);
-        }
-    }
     // k-stage t -> LDS stage t % NS; the loads of a stage are issued in two halves (h = 0, 1)
     constexpr int NLD0 = (NLD + 1) / 2;
     // Buffer addressing: a resource per operand (base pointer, no stride, no range limit), the per-lane
-    // 32-bit offset that never changes and a scalar offset that advances with the k-stage, so a load
-    // reads one address VGPR per lane and the loop carries no vector address arithmetic at all.
+    // 32-bit offset and a scalar offset that advances with the k-stage, so a load reads one address VGPR
+    // per lane and the loop carries no vector address arithmetic at all.
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a_base), 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(b_base), 0, -1, 0x00020000);
-    auto issue_half = [&](int t, int h) {
-        const int tt = t0 + (t < T ? t : T - 1);             // past the end: harmless reload into a free stage
+    auto issue_half = [&](const Unit& u, int t, int h) {
+        const int tt = u.t0 + (t < u.T ? t : u.T - 1);       // past the end: harmless reload into a free stage
         char* dst = smem + (t % NS) * STAGE + wave * 1024;
         const uint32_t sa = (uint32_t)tt * 64u, sb = (uint32_t)tt * (uint32_t)B_STEP;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             if ((i < NLD0) != (h == 0)) continue;
             if (16 * (4 * i) < BM)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, voff[i], sa, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, u.voff[i], sa, 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_ptr)(dst + i * 4096), 16, voff[i], sb, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_ptr)(dst + i * 4096), 16, u.voff[i], sb, 0, 0);
         }
     };
-    auto issue_stage = [&](int t) { issue_half(t, 0); issue_half(t, 1); };
+    auto issue_stage = [&](const Unit& u, int t) { issue_half(u, t, 0); issue_half(u, t, 1); };
 
     // ---- fragment addressing: lane (r = lane&31, kh = lane>>5) reads chunk 2s+kh of row base+r
     const int fr = lane & 31, fkh = lane >> 5;
@@ -668,6 +673,7 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
         off_a[s] = (wm * (BM / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
         off_b[s] = (BM + wn * (BN / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
     }
+    acc_t acc[FM][FN];
     u4_t fa[2][FM], fb[2][FN];
     auto read_frags = [&](int t, int s, int set) {
         const char* st = smem + (t % NS) * STAGE;
@@ -707,37 +713,82 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
         else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);      \
         else KMI_STAGE_BARRIER(0);                                         \
     } while (0)
-#pragma unroll
-    for (int t = 0; t < NS - 1; ++t) issue_stage(t);
     static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
-    KMI_STAGE_WAIT();
-    issue_half(NS - 1, 0);
-    read_frags(0, 0, 0);
-    for (int t = 0; t < T; ++t) {
-        // Slot (t-1) % NS was released by the previous barrier: it takes k-stage t+NS-1, half of the
-        // loads in each of the two MFMA blocks that follow that barrier, so the memory pipe sees one
-        // load per wave every few MFMAs instead of a burst.
-        read_frags(t, 1, 1);
-        issue_half(t + NS - 1, 1);
-        mfma_step(0);                                        // (t, step 0)
-        sched_interleave<NMF, NRD, 0, NLD - NLD0>();
-        __builtin_amdgcn_sched_barrier(0);
-        // stage t+1 has landed for every wave and stage t is fully in registers
+    // The epilogue's per-wave patches: the start of LDS in the one-tile form; the END of LDS in the
+    // persistent form (stage 3 and the last KiB of stage 2), which leaves stages 0 and 1 free to receive
+    // the next unit's first k-stages while this unit's results are written out.
+    constexpr int PATCH_BYTES = 4 * 32 * ((BN / 2) * 2 + 8);
+    constexpr int PATCH_OFF = PERSIST ? NS * STAGE - PATCH_BYTES : 0;
+    static_assert(!PERSIST || PATCH_OFF >= 2 * STAGE, "patches must stay clear of stages 0 and 1");
+
+    bool ahead = false;                                      // stages 0 and 1 of `cur` are already on their way
+    for (int vb = blockIdx.x;;) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+        if (PERSIST && ahead) {
+            // every wave has left the previous epilogue before stage 2 (whose end holds a patch) is refilled
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+            for (int t = 2; t < NS - 1; ++t) issue_stage(cur, t);
+        } else {
+#pragma unroll
+            for (int t = 0; t < NS - 1; ++t) issue_stage(cur, t);
+        }
+        // loads retire in issue order and the stores of a previous epilogue are older than every load
+        // counted here, so the same immediates hold for the first and for later units
         KMI_STAGE_WAIT();
-        read_frags(t + 1, 0, 0);                             // past the last stage: a harmless re-read
-        issue_half(t + NS, 0);
-        mfma_step(1);                                        // (t, step 1)
-        sched_interleave<NMF, NRD, 0, NLD0>();
-        __builtin_amdgcn_sched_barrier(0);
+        issue_half(cur, NS - 1, 0);
+        read_frags(0, 0, 0);
+        for (int t = 0; t < cur.T; ++t) {
+            // Slot (t-1) % NS was released by the previous barrier: it takes k-stage t+NS-1, half of the
+            // loads in each of the two MFMA blocks that follow that barrier, so the memory pipe sees one
+            // load per wave every few MFMAs instead of a burst.
+            read_frags(t, 1, 1);
+            issue_half(cur, t + NS - 1, 1);
+            mfma_step(0);                                    // (t, step 0)
+            sched_interleave<NMF, NRD, 0, NLD - NLD0>();
+            __builtin_amdgcn_sched_barrier(0);
+            // stage t+1 has landed for every wave and stage t is fully in registers
+            KMI_STAGE_WAIT();
+            read_frags(t + 1, 0, 0);                         // past the last stage: a harmless re-read
+            issue_half(cur, t + NS, 0);
+            mfma_step(1);                                    // (t, step 1)
+            sched_interleave<NMF, NRD, 0, NLD0>();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+        if constexpr (PERSIST) {
+            // the host uses this form without a split over K only
+            Unit nxt;
+            const bool more = vb + (int)gridDim.x < nvirt;
+            if (more) setup(vb + (int)gridDim.x, nxt);
+            auto start_next = [&]() {
+                if (more) {
+                    issue_stage(nxt, 0);
+                    issue_stage(nxt, 1);
+                }
+            };
+            if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next);
+            else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next);
+            if (!more) break;
+            cur = nxt;
+            ahead = true;
+            vb += (int)gridDim.x;
+        } else {
+            if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, cur.split, cur.m0, cur.n0, wave, lane);
+            else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane);
+            else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane);
+            break;
+        }
     }
 #undef KMI_STAGE_WAIT
-    // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 #undef KMI_STAGE_BARRIER
-
-    if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
-    else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
-    else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
 #endif
 }
 
@@ -772,6 +823,19 @@ int kmi_pick_splits(int M, int N, int K, int BM, int BN, int ktiles, const Works
     return s < 2 ? 1 : s;
 }
 
+// Compute units of the current device (0 if the query fails), asked once per device.
+static int cu_count() {
+    static std::atomic<int> cached[KMI_NOALLOC_MAX_DEVICES];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= KMI_NOALLOC_MAX_DEVICES) return 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 template <int KIND, int BM, int BN, bool TILED, int NS_ = 4>
 static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
@@ -797,7 +861,23 @@ static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st
     const int units = (int)(((long)a.K * (i8 ? 1 : 2)) >> (DIRECT ? 6 : 7));
     a.splits = whole ? kmi_pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units, ws) : 1;
     a.partial = a.splits > 1 ? ws.ptr : nullptr;
-    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
+    dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
+    if constexpr (DIRECT && TILED && BM == 256 && BN == 256 && NS == 4) {
+        // More tiles than CUs: one workgroup per CU walks the tiles (same order, same XCD per tile) and starts
+        // the next tile's loads before it writes the current one out.  Its weight offsets are 32-bit.
+        const int cus = cu_count();
+        if (a.splits == 1 && cus > 0 && (long)grid.x > cus && (long)a.N * a.K * (i8 ? 1 : 2) < (1L << 32)) {
+            void (*pfn)(GemmArgs) = gemm_direct_kernel<KIND, BM, BN, TILED, NS, true>;
+            static thread_local bool praised = false;
+            if (!praised) {
+                if (hipFuncSetAttribute(reinterpret_cast<const void*>(pfn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                    return kmi_set_error(KMI_E_LAUNCH, "gemm: cannot raise the dynamic LDS limit to %zu bytes", lds);
+                praised = true;
+            }
+            fn = pfn;
+            grid.x = (unsigned)cus;
+        }
+    }
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
         const long quads = (long)a.M * a.N / 4;

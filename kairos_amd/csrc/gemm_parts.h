@@ -132,9 +132,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
 // A wave converts one 32-row block at a time, writes it to its private LDS patch as fp16 [32][BN/2]
 // (8-byte writes, pitch padded by 8 bytes -> conflict free), and streams it out with 16-byte stores
 // in which 16 consecutive lanes cover 256 contiguous bytes of one output row.
-template <int KIND, int BM, int BN, bool HAS_BIAS, int FM, int FN, typename acc_t>
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+// `after_loads` runs once the per-column and per-row factors have arrived and before the first result leaves: a
+// persistent kernel starts the next tile's operand loads there, behind every load this epilogue waits for.
+template <int KIND, int BM, int BN, bool HAS_BIAS, int FM, int FN, typename acc_t, typename Hook = NoHook>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM][FN], char* smem, int m0, int n0,
-                                              int wave, int lane) {
+                                              int wave, int lane, Hook after_loads = Hook{}) {
     const int M = p.M, N = p.N;
     const int wm = wave >> 1, wn = wave & 1;
     const int c = lane & 31, hl = lane >> 5;
@@ -190,6 +195,27 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 as_i[i] = (float)p.ascales[m < M ? m : M - 1];
             }
         }
+        if constexpr (!std::is_same<Hook, NoHook>::value) {
+            // name every loaded factor as an operand, so the compiler places its waits for them here and
+            // none of its later waits can fall behind the loads that the hook starts
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(wsf[j][g][r]));
+                    }
+                    if constexpr (HAS_BIAS) asm volatile("" : "+v"(bs4[j][g]));
+                }
+            if constexpr (KIND == KIND_W8A8) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(as_i[i]));
+            }
+            asm volatile("" ::: "memory");
+            after_loads();
+            asm volatile("" ::: "memory");
+        }
         half_t* outp = static_cast<half_t*>(p.out);
         const bool wide = (N & 7) == 0;                  // 16-byte row segments stay aligned
 #pragma unroll
@@ -234,11 +260,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
 #pragma unroll
                 for (int k = 0; k < NK; ++k) {
                     const int m = mw + i * 32 + (k * 64 + lane) / CPR;
-#ifdef KMI_TEST_EPI_PLAIN
-                    if (m < M && n < N) *reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N) = v[k];
-#else
                     if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N));
-#endif
                 }
             } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
 #pragma unroll
@@ -279,11 +301,7 @@ __device__ __forceinline__ void sched_interleave() {
 // in column-major groups of GROUP_M tile rows, so the tiles resident on one XCD at a time form a
 // compact block that shares A row-panels and B column-panels in that XCD's L2.
 __device__ __forceinline__ void tile_of_block(int wg, int TM, int TN, int& tm, int& tn) {
-#ifdef KMI_TEST_GROUP_M
-    constexpr int XCDS = 8, GROUP_M = KMI_TEST_GROUP_M;
-#else
     constexpr int XCDS = 8, GROUP_M = 8;
-#endif
     const int total = TM * TN;
     const int xcd = wg % XCDS, q = wg / XCDS;
     const int base = total / XCDS, rem = total % XCDS;

@@ -346,6 +346,46 @@ def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
     assert torch.equal(acc, again) and torch.equal(acc, ops.w8a8_gemm_acc_i32(a8, w8, N))
 
 
+@pytest.mark.parametrize("K", [128, 384])
+def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K):
+    """More 256 x 256 tiles than compute units (9 x 31 = 279, ragged in M and N): the tiled-weight W8A8 and fp16 GEMMs
+    then run one workgroup per CU that walks the tiles and starts a tile's first loads while the previous one is
+    written out.  K = 128 is shorter than the load pipeline.  Outputs equal the 128-row-tile kernel's bit for bit
+    (same accumulation order) and the oracle's on sampled rows, with and without a bias."""
+    M, N = 2100, 7808
+    p = prep(N, K, seed=K)
+    x = O.synth_acts(M, K, seed=K + 1)
+    a8_np, sx_np = O.quant_act_i8(x)
+    bias_np = np.random.default_rng(K).standard_normal(N).astype(np.float16)
+    rows = np.array([0, 1, 255, 256, 2047, 2048, 2099])
+    _, ref8 = O.gemm_w8a8(a8_np[rows], p["w8"], p["scales_1"], sx_np[rows])
+    ref8_b = (ref8.astype(np.float32) + bias_np.astype(np.float32)).astype(np.float16)
+    w8_t = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    ops.dequant_interleaved_int4_to_int8(w8_t, dev(p["qweight"]), dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), 128, tiled=True)
+    w16_t = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    ops.dequant_interleaved_int4_to_fp16(w16_t, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), 128, tiled=True)
+    a8, sx, xd, bias, s1 = dev(a8_np), dev(sx_np), dev(x), dev(bias_np), dev(p["scales_1"])
+    got = {}
+    for tile in (256, 128):
+        ops.force_gemm_tile(tile)
+        ops.force_gemm_splits(1)
+        try:
+            o8 = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            o8b = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            ops.w8a8_gemm_forward(a8, w8_t, s1, sx, o8, tiled=True)
+            ops.w8a8_gemm_forward(a8, w8_t, s1, sx, o8b, bias=bias, tiled=True)
+            got[tile] = (o8, o8b, ops.f16_gemm_forward(xd, w16_t, N, tiled=True),
+                         ops.f16_gemm_forward(xd, w16_t, N, bias=bias, tiled=True))
+        finally:
+            ops.force_gemm_tile(0)
+            ops.force_gemm_splits(0)
+    for a, b in zip(got[256], got[128]):
+        assert torch.equal(a, b)
+    assert_same_bits(host(got[256][0])[rows], ref8)
+    assert_same_bits(host(got[256][1])[rows], ref8_b)
+    assert O.max_abs_rel(host(got[256][2])[rows], O.gemm_f16(x[rows], p["w16"])) < 2e-3
+
+
 @pytest.mark.parametrize("tile", [64, 128, 256])
 @pytest.mark.parametrize("M", GEMM_M)
 def test_gemm_w4a16_f16_w8a16(ops, M, tile):
