@@ -19,7 +19,7 @@ import json
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-HASHED_SOURCES = ["csrc/gemm_mfma.hip", "csrc/kmi_common.h"]
+HASHED_SOURCES = ["csrc/gemm_mfma.hip", "csrc/gemm_parts.h", "csrc/kmi_common.h"]
 COPY_BYTES = 1 << 30
 
 
