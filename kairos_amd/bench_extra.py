@@ -22,8 +22,8 @@ import torch
 
 from . import ops
 from .act_matching import MatchedRMSNorm, MatchedSiluMul
-from .dynamic_linear import COMP_TYPE_NAME, DynamicLinear
-from .perf_profiler import Profiler
+from .dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear     # version 2: the same classes plus the W4A8 lane
+from .perf_profiler_v2 import Profiler
 from .temp_cache import TempCache
 
 HBM = 8.0e12
@@ -580,7 +580,7 @@ def main(argv=None):
         sys.exit("bench_extra: needs a GPU (the HIP library is the only compute path)")
     if args.cmd == "decoder" and args.lut is None:
         import os
-        args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x") + "/"
+        args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x_v2") + "/"
     res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
