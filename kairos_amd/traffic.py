@@ -1,10 +1,10 @@
 """HBM <-> L2 traffic of one kernel family of `bench.py`, from two rocprofv3 counter runs.
 
     cd /tmp && export TMPDIR=/tmp && cd <repo>
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -o b -- python3 bench.py --only-label 'gemm_w8a8[256]' --steps 3 --warmup 1 --calib-copy --calls-json gpurun_out/pmc_calls.json
-    rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o b -- python3 bench.py --only-label 'gemm_w8a8[256]' --steps 3 --warmup 1 --calib-copy
-    python3 -m kairos_amd.traffic --label 'gemm_w8a8[256]' --kernel gemm_direct_kernel --fetch gpurun_out/pmc_fetch/b_counter_collection.csv \
-        --write gpurun_out/pmc_write/b_counter_collection.csv --calls-json gpurun_out/pmc_calls.json --out profiles/bench_llama3_8b_traffic.json
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d prof_out/pmc_fetch -o b -- python3 bench.py --only-label 'gemm_w8a8[256]' --steps 3 --warmup 1 --calib-copy --calls-json prof_out/pmc_calls.json
+    rocprofv3 --pmc WRITE_SIZE --output-format csv -d prof_out/pmc_write -o b -- python3 bench.py --only-label 'gemm_w8a8[256]' --steps 3 --warmup 1 --calib-copy
+    python3 -m kairos_amd.traffic --label 'gemm_w8a8[256]' --kernel gemm_direct_kernel --fetch prof_out/pmc_fetch/b_counter_collection.csv \
+        --write prof_out/pmc_write/b_counter_collection.csv --calls-json prof_out/pmc_calls.json --out profiles/bench_llama3_8b_traffic.json
 
 `bench.py --only-label L` runs only the calls of the step that the benchmark books under label L, so every dispatch of
 the kernel family in the counter files belongs to L (a call may be two dispatches: head and tail launch).  `--calib-copy`
