@@ -79,8 +79,13 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-template <int KIND, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_w4a8_kernel(GemmArgs p) {
+// KH = 2: two wave quartets per workgroup.  Each is the whole pipeline below on its own half of the workgroup's K range
+// with its own LDS ring; they share nothing but the barriers, so on every SIMD one wave's decode instructions issue under
+// the other's MFMAs -- what two workgroups per CU do for each other, without a second output tile or partial sums in
+// memory.  Their int32 accumulators meet in LDS at the end (integers: the order does not matter).  Small tiles only:
+// two waves per SIMD leave 256 registers each.
+template <int KIND, int BM, int BN, int KH = 1>
+__global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     static_assert(KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC, "int8 accumulation");
     constexpr int NS = 4;
@@ -93,9 +98,12 @@ __global__ __launch_bounds__(256) void gemm_w4a8_kernel(GemmArgs p) {
     static_assert(BM % 64 == 0 && (BN == 128 || BN == 256) && NLA >= 2, "tile shapes this staging scheme covers");
     using acc_t = i16_t;
 
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    static_assert(KH == 1 || (KH == 2 && FM * FN < 16), "two quartets: accumulators in VGPRs, 256 registers per wave");
+    extern __shared__ __attribute__((aligned(16))) char smem_all[];
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & 255;                       // index inside the quartet
+    const int kq = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    char* const smem = smem_all + kq * (NS * STAGE);         // this quartet's ring
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
@@ -105,9 +113,10 @@ __global__ __launch_bounds__(256) void gemm_w4a8_kernel(GemmArgs p) {
     tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
     const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
     const int T_all = K >> 6;                                // 64-byte stages along K (K % 128 == 0: even)
-    const int t_per = (((T_all + p.splits - 1) / p.splits) + 1) & ~1;   // whole groups per split
-    const int t0 = split * t_per;
-    const int T = (t0 + t_per <= T_all) ? t_per : T_all - t0;            // even, >= 2 (the host leaves no empty split)
+    const int t_per = (((T_all + p.splits - 1) / p.splits) + 2 * KH - 1) / (2 * KH) * (2 * KH);   // whole groups per split and quartet
+    const int t_split = (split * t_per + t_per <= T_all) ? t_per : T_all - split * t_per;   // even, >= 2 (no empty split)
+    const int T = t_split / KH;                              // two quartets: the host keeps this even as well
+    const int t0 = split * t_per + kq * T;
 
     acc_t acc[FM][FN];
 #pragma unroll
@@ -328,6 +337,27 @@ __global__ __launch_bounds__(256) void gemm_w4a8_kernel(GemmArgs p) {
     // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
+    if constexpr (KH > 1) {                                  // quartet 1 hands its accumulators to quartet 0 and leaves
+        constexpr int RED_OFF = 32 * 1024;                   // clear of the epilogue's patches at the start of LDS
+        static_assert(4 * 32 * ((BN / 2) * 2 + 8) <= RED_OFF && RED_OFF + FM * FN * 16 * 256 * 4 <= KH * NS * STAGE, "LDS layout of the hand-over");
+        int* red = reinterpret_cast<int*>(smem_all + RED_OFF);
+        if (kq == 1) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) red[((i * FN + j) * 16 + e) * 256 + tid] = acc[i][j][e];
+        }
+        __syncthreads();
+        if (kq == 1) return;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] += red[((i * FN + j) * 16 + e) * 256 + tid];
+    }
     if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
     else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
     else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
@@ -335,14 +365,14 @@ __global__ __launch_bounds__(256) void gemm_w4a8_kernel(GemmArgs p) {
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-template <int KIND, int BM, int BN>
+template <int KIND, int BM, int BN, int KH = 1>
 static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const Workspace ws = (a.n_begin == 0 && a.n_cols == a.N) ? ws_in : Workspace{nullptr, 0};   // column ranges: no split over K
-    constexpr size_t lds = (size_t)4 * (BM + BN) * 64;
-    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN>;
+    constexpr size_t lds = (size_t)KH * 4 * (BM + BN) * 64;
+    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN, KH>;
     static thread_local bool raised = false;                 // per instantiation, per thread
     if (lds > 64 * 1024 && !raised) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -352,13 +382,15 @@ static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t
     // K splits as for the W8A8 lane, in whole 128-wide groups (two stages), no empty split
     const int stages = a.K >> 6;
     int s = kmi_pick_splits(a.M, a.N, a.K, BM, BN, a.K >> 7, ws);
+    constexpr int UNIT = 2 * KH;                             // stages per split: whole groups for every quartet
     if (s > 1) {
-        const int per = (((stages + s - 1) / s) + 1) & ~1;
+        const int per = (((stages + s - 1) / s) + UNIT - 1) / UNIT * UNIT;
         s = (stages + per - 1) / per;
     }
+    if (KH == 2 && (stages % UNIT != 0)) return kmi_set_error(KMI_E_SHAPE, "gemm_w4a8: two quartets need K %% 256 == 0 (K=%d)", a.K);
     a.splits = s < 2 ? 1 : s;
     a.partial = a.splits > 1 ? ws.ptr : nullptr;
-    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
+    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256 * KH);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
         const long quads = (long)a.M * a.N / 4;
@@ -388,6 +420,7 @@ static int w4a8_head_cols(int M, int N) {
 static int w4a8_tile(int M, int N, int K) {
     const int forced = kmi_forced_tile();
     if (forced == 128 || forced == 192 || forced == 256) return forced;
+    if (forced == 130) return (K % 256 == 0) ? 130 : 128;    // 128 x 128 tile, two wave quartets per workgroup
     if (forced == 448) return w4a8_head_cols(M, N) > 0 ? 448 : 256;
     const Workspace roomy{reinterpret_cast<void*>(16), (size_t)64 << 20};
     const double t256 = 69.5 * (double)K / 4096.0;
@@ -409,7 +442,14 @@ static int w4a8_tile(int M, int N, int K) {
         const long tail = (long)(TN - head) * TM * 2;
         c448 = ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256 + 2.0;
     }
-    if (c128 <= c192 && c128 <= c256 && c128 <= c448) return 128;
+    if (c128 <= c192 && c128 <= c256 && c128 <= c448) {
+        // At most one workgroup per CU: two wave quartets per workgroup, each on half of the workgroup's K range
+        // (28672 columns M=128: 28.0 against 32.5 us; 6144 columns M=512: 24.8 against 29.6; 4096 x 14336 M=256 with
+        // four splits: 33.1 against 35.5; level elsewhere).  More workgroups than CUs overlap each other already.
+        const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+        const int sp = kmi_pick_splits(M, N, K, 128, 128, K >> 7, roomy);
+        return (K % 256 == 0 && tiles * sp <= 256) ? 130 : 128;
+    }
     if (c448 <= c192 && c448 <= c256) return 448;
     return c192 <= c256 ? 192 : 256;
 }
@@ -434,7 +474,8 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
         if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128>(a, ws, st, head, a.N - head);
     } else {
         rc = tile == 256 ? launch_w4a8<KIND, 256, 256>(a, ws, st)
-           : tile == 192 ? launch_w4a8<KIND, 256, 128>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
+           : tile == 192 ? launch_w4a8<KIND, 256, 128>(a, ws, st)
+           : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
     }
     if (rc != KMI_OK) return rc;
     return kmi_check_launch(fn);
