@@ -37,6 +37,13 @@ __device__ __forceinline__ uint32_t w4a8_table_word(half_t s, half_t z) {
     return pack_i8x4(pk_fma(q01, s2, z2), pk_fma(q23, s2, z2));
 }
 
+// The same for the nibble values held in q01 / q23 (four consecutive values as fp16 pairs): the form used when two
+// threads share a weight row and each builds half of the row's table.
+__device__ __forceinline__ uint32_t w4a8_table_word_of(h2_t q01, h2_t q23, half_t s, half_t z) {
+    const h2_t s2 = {s, s}, z2 = {z, z};
+    return pack_i8x4(pk_fma(q01, s2, z2), pk_fma(q23, s2, z2));
+}
+
 // Four nibbles (`idx3`: their low three bits, one per byte; `sel_hi`: 0x03020100 + 4 * bit 3, one per byte) -> four
 // table bytes.
 __device__ __forceinline__ uint32_t w4a8_lookup(const uint32_t (&L)[4], uint32_t idx3, uint32_t sel_hi) {
@@ -185,12 +192,32 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
     const W4a8Masks wm4 = w4a8_masks();
     uint32_t xy[4];
     u4_t dq;
+    // BN = 128: the two threads of a row (lanes 2r, 2r+1) need the same table; each builds the half for the nibble
+    // values 8*hsel .. 8*hsel+7 and gets the other half from its neighbour with a lane swap inside the quad.
+    h2_t tq[4];                                              // the eight nibble values of this thread's half, as fp16 pairs
+    uint32_t town[2], tnbr[2];
+    if constexpr (CPT == 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tq[i] = h2_t{(half_t)(float)(8 * hsel + 2 * i), (half_t)(float)(8 * hsel + 2 * i + 1)};
+    }
     auto work_item = [&](auto sp, auto gn, auto with_table, auto item, int slot) {
         constexpr int SPv = decltype(sp)::value, GNv = decltype(gn)::value, IT = decltype(item)::value;
         constexpr int NT = decltype(with_table)::value ? 4 : 0;
         if constexpr (IT < NT) {
             const half_t sc = __builtin_bit_cast(half_t, sraw[GNv]), zc = __builtin_bit_cast(half_t, zraw[GNv]);
-            L[IT] = w4a8_table_word<IT>(sc, zc);
+            if constexpr (CPT == 2) {
+                L[IT] = w4a8_table_word<IT>(sc, zc);
+            } else if constexpr (IT < 2) {
+                town[IT] = w4a8_table_word_of(tq[2 * IT], tq[2 * IT + 1], sc, zc);
+            } else if constexpr (IT == 2) {                  // quad_perm [1, 0, 3, 2]: the other thread of the row
+                tnbr[0] = (uint32_t)__builtin_amdgcn_mov_dpp((int)town[0], 0xB1, 0xF, 0xF, true);
+                tnbr[1] = (uint32_t)__builtin_amdgcn_mov_dpp((int)town[1], 0xB1, 0xF, 0xF, true);
+            } else {
+                L[0] = hsel ? tnbr[0] : town[0];
+                L[1] = hsel ? tnbr[1] : town[1];
+                L[2] = hsel ? town[0] : tnbr[0];
+                L[3] = hsel ? town[1] : tnbr[1];
+            }
         } else if constexpr (IT < NT + 9 * CPT) {
             constexpr int J = (IT - NT) / 9, ST = (IT - NT) % 9;
             if constexpr (ST == 0) {
@@ -423,32 +450,43 @@ static int w4a8_tile(int M, int N, int K) {
     if (forced == 130) return (K % 256 == 0) ? 130 : 128;    // 128 x 128 tile, two wave quartets per workgroup
     if (forced == 448) return w4a8_head_cols(M, N) > 0 ? 448 : 256;
     const Workspace roomy{reinterpret_cast<void*>(16), (size_t)64 << 20};
-    const double t256 = 69.5 * (double)K / 4096.0;
+    const double fixed = 6.0;                                // launch, pipeline fill, epilogue: paid once per launch, split or not
+    const double t256 = 63.5 * (double)K / 4096.0;           // + fixed = 69.5 us at K = 4096
     auto cost = [&](int bm, int bn, double unit_alone, double unit_shared, int shared_cap) {
         const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         const int s = kmi_pick_splits(M, N, K, bm, bn, K >> 7, roomy);
         const long w = tiles * s;
         const double rounds_t = w <= 256 ? unit_alone : (double)((w + shared_cap - 1) / shared_cap) * unit_shared;
-        double us = rounds_t * t256 / s;
+        double us = fixed + rounds_t * t256 / s;
         if (s > 1) us += (double)(s + 1) * (double)M * (double)N * 4.0 / 4.0e6 + 3.0;
         return us;
     };
-    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.59, 0.59, 256), c128 = cost(128, 128, 0.50, 0.67, 512);
+    // 128 x 128 alone on a CU: 0.45 with one wave quartet.  With two (selector 130, needs K % 256 == 0, at most one
+    // workgroup per CU) the time is a fixed ~7 us + 0.265 us per 64-byte stage, rising to 0.315 as the last CUs fill
+    // (4096 x 4096 M=128: 17.7 us, M=1024: 26.4; 4096 x 14336 M=1024: 77.3 against 91.8 with split 256 x 256 tiles).
+    const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const int s128 = kmi_pick_splits(M, N, K, 128, 128, K >> 7, roomy);
+    const bool two_quartets = (K % 256 == 0) && tiles128 * s128 <= 256;
+    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.59, 0.59, 256);
+    double c128 = cost(128, 128, 0.45, 0.67, 512);
+    if (two_quartets) {
+        const double w = (double)(tiles128 * s128);
+        c128 = 7.0 + (0.265 + (w > 192.0 ? 0.05 * (w - 192.0) / 64.0 : 0.0)) * (double)(K >> 6) / s128;
+        if (s128 > 1) c128 += (double)(s128 + 1) * (double)M * (double)N * 4.0 / 4.0e6 + 3.0;
+    }
     // 256 x 256 tiles in whole rounds of 256 and the columns of the thin last round as 256 x 128 tiles in a second
     // launch (selector 448): 2048 x 28672 is 896 tiles = 3.5 rounds -> 3 rounds + one round of half-size tiles.
     double c448 = 1e30;
     if (w4a8_head_cols(M, N) > 0) {
         const int TM = (M + 255) / 256, TN = (N + 255) / 256, head = w4a8_head_cols(M, N);
         const long tail = (long)(TN - head) * TM * 2;
-        c448 = ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256 + 2.0;
+        c448 = 2.0 * fixed + ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256;
     }
     if (c128 <= c192 && c128 <= c256 && c128 <= c448) {
         // At most one workgroup per CU: two wave quartets per workgroup, each on half of the workgroup's K range
         // (28672 columns M=128: 28.0 against 32.5 us; 6144 columns M=512: 24.8 against 29.6; 4096 x 14336 M=256 with
         // four splits: 33.1 against 35.5; level elsewhere).  More workgroups than CUs overlap each other already.
-        const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-        const int sp = kmi_pick_splits(M, N, K, 128, 128, K >> 7, roomy);
-        return (K % 256 == 0 && tiles * sp <= 256) ? 130 : 128;
+        return two_quartets ? 130 : 128;
     }
     if (c448 <= c192 && c448 <= c256) return 448;
     return c192 <= c256 ? 192 : 256;
