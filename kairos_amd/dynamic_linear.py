@@ -20,6 +20,7 @@ import itertools
 import torch
 
 from . import ops
+from .ops import GEMV_MAX_M as _GEMV_MAX_M, _gemv_workspaces, _raw_stream
 from .temp_cache import default_cache
 from .weight_prep import calculate_zeros_width, prepare_linear_weight
 
@@ -145,8 +146,40 @@ class DynamicLinear(torch.nn.Module):
             self.comp_type = comp
         return self.comp_type
 
-    @torch.no_grad()
     def forward(self, input) -> torch.Tensor:
+        # Decode-sized calls are host-bound (the kernels take 5-13 us, a Python call with a launch about as long), so
+        # the small-M lane is served right here: one allocation, one C call, cached pointers, no context managers.
+        # Nothing on it records autograd history (the output is a fresh tensor filled by the library).
+        if type(input) is torch.Tensor:
+            shape = input.shape
+            m = input.numel() // shape[-1]
+            if m != self.pre_m:
+                self._select(m)
+            if (self.comp_type == _W4A16_GEMV and m <= _GEMV_MAX_M and ops._tracer is None
+                    and input.dtype is torch.float16 and input.is_cuda and input.is_contiguous()):
+                ptrs = self._decode_ptrs
+                if ptrs is None or ptrs[0] != self._buffers['qweight'].data_ptr():
+                    ptrs = self._decode_ptrs = self._decode_pointers(input.device)
+                out = torch.empty(shape[:-1] + (ptrs[6],), dtype=torch.float16, device=input.device)
+                st = _raw_stream(ptrs[5]) if _raw_stream is not None else ops._stream()
+                ws = _gemv_workspaces.get((ptrs[5], st))
+                if ws is None:
+                    ws = ops.gemv_workspace_for(input.device, st)
+                rc = ptrs[4](out.data_ptr(), input.data_ptr(), ptrs[0], ptrs[1], ptrs[2], ptrs[3], m, ptrs[6], ptrs[7], ptrs[8],
+                             ws.data_ptr(), ws.numel(), st)
+                if rc < 0:
+                    ops._lib.check(rc)
+                return out
+        return self._forward_any(input)
+
+    def _decode_pointers(self, device):
+        N, K = self.shape
+        return (self.qweight.data_ptr(), self.scales.data_ptr(), self.scaled_zeros.data_ptr(),
+                0 if self.bias is None else self.bias.data_ptr(), ops._lib.load().kmi_gemv_w4a16, device.index or 0,
+                N, K, self.group_size)
+
+    @torch.no_grad()
+    def _forward_any(self, input) -> torch.Tensor:
         shape = input.shape
         K = shape[-1]
         m = input.numel() // K
@@ -160,30 +193,7 @@ class DynamicLinear(torch.nn.Module):
                 raise ValueError("the matched activation holds no fp16 form, but this layer's lane for "
                                  f"{m} tokens (id {self.comp_type}) needs one")
             input = input.f16
-        if self.comp_type == _W4A16_GEMV and m <= ops.GEMV_MAX_M and ops._tracer is None:
-            return self._forward_decode(input, shape, m)
         return self._forward(input.reshape(-1, K), m, self.comp_type).reshape(*shape[:-1], -1)
-
-    def _forward_decode(self, input, shape, m):
-        """Decode-sized calls are host-bound: one allocation, one C call, cached pointers."""
-        if input.dtype is not torch.float16 or not input.is_cuda or not input.is_contiguous():
-            return self._forward(input.reshape(-1, shape[-1]), m, self.comp_type).reshape(*shape[:-1], -1)
-        ptrs = self._decode_ptrs
-        if ptrs is None or ptrs[0] != self.qweight.data_ptr():
-            ptrs = self._decode_ptrs = (self.qweight.data_ptr(), self.scales.data_ptr(), self.scaled_zeros.data_ptr(),
-                                        0 if self.bias is None else self.bias.data_ptr(),
-                                        ops._lib.load().kmi_gemv_w4a16, input.device.index or 0)
-        N, K = self.shape
-        out = torch.empty(shape[:-1] + (N,), dtype=torch.float16, device=input.device)
-        st = ops._raw_stream(ptrs[5]) if ops._raw_stream is not None else ops._stream()
-        ws = ops._gemv_workspaces.get((ptrs[5], st))
-        if ws is None:
-            ws = ops.gemv_workspace_for(input.device, st)
-        rc = ptrs[4](out.data_ptr(), input.data_ptr(), ptrs[0], ptrs[1], ptrs[2], ptrs[3], m, N, K, self.group_size,
-                     ws.data_ptr(), ws.numel(), st)
-        if rc < 0:
-            ops._lib.check(rc)
-        return out
 
     def _w8a8(self, x, int_x, scale_x):
         """The W8A8 lane on fp16 activations x [m, K], or on activations that arrive quantised (x None)."""
