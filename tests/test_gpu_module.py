@@ -86,6 +86,53 @@ def test_forward_uses_lut_and_counts_switches(gpu, tmp_path):
         DynamicLinear.prof = old
 
 
+def test_small_m_call_in_forward_agrees_with_the_general_path(gpu):
+    """forward() serves decode-sized fp16 calls itself (one allocation, one C call).  Inputs it does not take -- a
+    strided view, a tracer installed, a replaced weight tensor -- go the general way; all of them give the same bits,
+    with and without a bias, and the cached pointers follow a weight that was replaced."""
+    from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
+    from kairos.perf_profiler import Profiler
+    from kairos_amd import ops
+    N, K = 256, 512
+    prof = Profiler([(N, K)])
+    prof.record_best_comp((N, K), 64, 'w4a16_gemv')
+    prof.record_best_comp((N, K), 4096, 'w8a8')
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        for bias in (False, True):
+            lin, w = make_linear(N, K, bias)
+            dl = DynamicLinear.from_module(lin.cuda(), 'cuda')
+            x = torch.from_numpy(O.synth_acts(6, K, seed=3)).cuda().reshape(2, 3, K)
+            fast = dl(x)
+            assert fast.shape == (2, 3, N) and dl.comp_type == COMP_TYPE_NAME['w4a16_gemv'] and dl._decode_ptrs is not None
+            general = dl._forward(x.reshape(-1, K), 6, dl.comp_type).reshape(2, 3, N)
+            assert torch.equal(fast, general)
+            wide = torch.zeros((2, 3, 2 * K), dtype=torch.float16, device='cuda')
+            wide[..., :K] = x
+            assert not wide[..., :K].is_contiguous() and torch.equal(dl(wide[..., :K]), fast)      # strided view
+            calls = []
+
+            class Tracer:
+                def begin(self, name, M, N_, K_):
+                    calls.append((name, M, N_, K_))
+
+                def end(self):
+                    pass
+            ops.set_tracer(Tracer())
+            try:
+                assert torch.equal(dl(x), fast) and calls == [("gemv_w4a16", 6, N, K)]            # traced: general path
+            finally:
+                ops.set_tracer(None)
+            # a replaced weight: the cached raw pointers must not outlive it
+            lin2, _ = make_linear(N, K, bias, seed=99)
+            other = DynamicLinear.from_module(lin2.cuda(), 'cuda')
+            dl.load_state_dict(other.state_dict())
+            assert torch.equal(dl(x), other(x))
+    finally:
+        DynamicLinear.prof = old
+
+
 def test_temp_cache_reuse_and_bound(gpu):
     from kairos.dynamic_linear import COMP_TYPE_NAME, DynamicLinear
     from kairos_amd.temp_cache import TempCache
