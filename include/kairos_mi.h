@@ -237,7 +237,8 @@ int kmi_gemm_w4a16_noalloc(void* out_f16, const void* x_f16, const void* qweight
                            const void* scaled_zeros, const void* bias, int M, int N, int K, int G, void* stream);
 
 /* Host-only queries of the automatic choices (no GPU work).
- * kmi_gemm_pick_tile: the workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns) of the W8A8 lane for an
+ * kmi_gemm_pick_tile: the workgroup tile (64, 128 or 256 rows; 192 = 256 rows x 128 columns; 320 = 256 rows x 192
+ *   columns, used with tiled weights only -- row-major operands run 256 x 256 instead) of the W8A8 lane for an
  *   M x N x K product.  With the 256 tile the library may run the columns of a thin last round of tiles with the 128
  *   tile in a second launch on the same stream (same results).
  * kmi_gemm_w4a16_wp_rows: rows per tile (32, 64, 128) of the small-M variant kmi_gemm_w4a16 uses (weights decoded in

@@ -613,7 +613,9 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
         u.n0 = p.n_begin + tn * BN;
         u.t0 = u.split * t_per;                              // this unit covers stages t0 .. t0+T-1
         u.T = (u.t0 + t_per <= T_all) ? t_per : T_all - u.t0;
-        const long fold = (TILED_B && PERSIST) ? (long)(u.n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64) : 0;
+        // FOLD: the weight strip of the tile goes into the per-lane offsets (several tiles per workgroup, or tiles
+        // whose width is not a whole number of 128-row strips, so that a tile may start in the middle of one)
+        constexpr bool FOLD = TILED_B && (PERSIST || (BN % KMI_TILE_N) != 0);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int row = 16 * (4 * i + wave) + (lane >> 2);
@@ -624,10 +626,13 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
                 m = m < M ? m : M - 1;
                 u.voff[i] = (uint32_t)((long)m * row_bytes + c * 16);
             } else if constexpr (TILED_B) {
+                // 16-row groups never straddle a strip (tiles start at multiples of 64 columns); the stored swizzle
+                // depends on the row inside the strip, which equals the row inside the tile modulo 16
                 const int rb = row - BM;
-                int strip = rb >> 7;
-                if (u.n0 + strip * KMI_TILE_N >= N) strip = 0;
-                u.voff[i] = (uint32_t)(fold + (long)strip * T_all * (KMI_TILE_N * 64) + (rb & 127) * 64 + pc * 16);
+                const int base_n = FOLD ? 0 : (u.n0 / KMI_TILE_N) * KMI_TILE_N;   // first column of the strip at the resource's base
+                int nrel = u.n0 - base_n + rb;                                     // this row's column relative to it
+                if (base_n + nrel >= N) nrel = ((u.n0 - base_n) & ~(KMI_TILE_N - 1)) + (rb & (KMI_TILE_N - 1));   // ragged last tile: the (valid) strip of n0; stores are masked
+                u.voff[i] = (uint32_t)((long)(nrel >> 7) * T_all * (KMI_TILE_N * 64) + (nrel & 127) * 64 + pc * 16);
             } else {
                 int n = u.n0 + row - BM;
                 n = n < N ? n : N - 1;
@@ -640,7 +645,7 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
 
     const char* a_base = static_cast<const char*>(p.a);
     const char* b_base = static_cast<const char*>(p.b);
-    if constexpr (TILED_B && !PERSIST) b_base += (long)(cur.n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64);
+    if constexpr (TILED_B && !(PERSIST || (BN % KMI_TILE_N) != 0)) b_base += (long)(cur.n0 / KMI_TILE_N) * T_all * (KMI_TILE_N * 64);
     constexpr long B_STEP = TILED_B ? KMI_TILE_N * 64 : 64;
     // k-stage t -> LDS stage t % NS; the loads of a stage are issued in two halves (h = 0, 1)
     constexpr int NLD0 = (NLD + 1) / 2;
@@ -707,6 +712,7 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
 #define KMI_STAGE_WAIT()                                                   \
     do {                                                                   \
         if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);         \
+        else if constexpr (NLD * (NS - 2) == 14) KMI_STAGE_BARRIER(14);    \
         else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);      \
         else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);      \
         else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);      \
@@ -714,6 +720,8 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
         else KMI_STAGE_BARRIER(0);                                         \
     } while (0)
     static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
+    static_assert(NLD * (NS - 2) == 16 || NLD * (NS - 2) == 14 || NLD * (NS - 2) == 8 || NLD * (NS - 2) == 6 || NLD * (NS - 2) == 4 ||
+                  NLD * (NS - 2) == 3, "no wait immediate for this tile and depth");
     // The epilogue's per-wave patches: the start of LDS in the one-tile form; the END of LDS in the
     // persistent form (stage 3 and the last KiB of stage 2), which leaves stages 0 and 1 free to receive
     // the next unit's first k-stages while this unit's results are written out.
@@ -862,7 +870,7 @@ static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st
     a.splits = whole ? kmi_pick_splits(a.M, a.N, a.K, BM, BN, DIRECT ? units / 2 : units, ws) : 1;
     a.partial = a.splits > 1 ? ws.ptr : nullptr;
     dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256);
-    if constexpr (DIRECT && TILED && BM == 256 && BN == 256 && NS == 4) {
+    if constexpr (DIRECT && TILED && BM == 256 && (BN == 256 || BN == 192) && NS == 4) {
         // More tiles than CUs: one workgroup per CU walks the tiles (same order, same XCD per tile) and starts
         // the next tile's loads before it writes the current one out.  Its weight offsets are 32-bit.
         const int cus = cu_count();
@@ -946,7 +954,13 @@ static int pick_tile(int M, int N, long row_bytes) {
     long split = 256 / wgs(256, 256);
     if (split > row_bytes / 9000) split = row_bytes / 9000;
     if (split < 1) split = 1;
-    if (M > 128 && wgs(256, 256) * split >= 144) return 256;
+    if (M > 128 && wgs(256, 256) * split >= 144) {
+        // One round either way: 256 x 192 tiles (N a multiple of 192 and of the 128-row weight strips; selector 320,
+        // tiled weights only) put the same output on more CUs with less work each.  The narrower tile is less efficient
+        // per MFMA, so the gain is small: 2048 x 6144 x 4096 51.9 against 54.9 us, 2048 x 4608 x 3584 37.9 against 45.1.
+        if (split == 1 && N % 384 == 0 && wgs(256, 192) <= 256 && wgs(256, 256) < wgs(256, 192)) return 320;
+        return 256;
+    }
     // too few 256 x 256 tiles for the CUs, yet the rows are too short to split: 256 x 128 tiles, two workgroups per CU
     // (selector 192), when they come to 192..256 (2048 x 4096 x 14336: 119 against 130 us with 128 x 128 tiles and 134
     // with 256 x 256; 1536 x 4096 x 14336: 95 against 106; on long rows the split 256 tile wins: 1024 x 8192 x 28672)
@@ -990,7 +1004,7 @@ extern "C" int kmi_gemm_w4a16_wp_rows(int M, int N, int K) { return pick_wp(M, N
 
 template <int KIND, bool TILED>
 static int dispatch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t st, int force_tile) {
-    const int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N, (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC) ? (long)a.K : 0);
+    int tile = force_tile > 0 ? force_tile : pick_tile(a.M, a.N, (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC) ? (long)a.K : 0);
     if constexpr (KIND == KIND_W4A16) {
         // selectors 1032 / 1064 / 1128 force the wave-private-weights kernel with 32 / 64 / 128 rows per tile
         if (tile == 1032) return launch_w4a16_wp<32>(a, ws, st);
@@ -1008,6 +1022,8 @@ static int dispatch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t st,
             if (c.rows == 128) return launch_w4a16_wp<128, 1>(a, ws, st);
         }
     }
+    if (tile == 320 && !(TILED && (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16)))
+        tile = 256;                                          // row-major operands and the other kinds: 256 x 256 as before
     if (tile == 256 && force_tile == 0) {
         // Round quantisation: TM x TN tiles run in rounds of 256 (one workgroup per CU).  When the last
         // round would be at most ~60 % full, the columns it would cover are run with the 128x128 tile
@@ -1024,6 +1040,9 @@ static int dispatch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t st,
     }
     switch (tile) {
         case 256: return launch_gemm<KIND, 256, 256, TILED>(a, ws, st);
+        case 320:                                        // 256 rows x 192 columns (tiled weights): N = 6144 in whole tiles
+            if constexpr (TILED && (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16)) return launch_gemm<KIND, 256, 192, TILED>(a, ws, st);
+            break;
         case 192:                                        // 256 rows x 128 columns, three stages, two workgroups per CU
             if constexpr (KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC || KIND == KIND_F16) return launch_gemm<KIND, 256, 128, TILED, 3>(a, ws, st);
             break;
@@ -1192,7 +1211,7 @@ extern "C" int kmi_gemm_splits_for(int lane, int M, int N, int K, size_t workspa
         const int head_cols = (tiles - rem) / TM;
         if (tiles > 256 && rem > 0 && head_cols > 0 && (TN - head_cols) * TM <= 160) return 1;
     }
-    const int BM = tile == 64 ? 64 : tile == 128 ? 128 : 256, BN = (tile == 256) ? 256 : 128;
+    const int BM = tile == 64 ? 64 : tile == 128 ? 128 : 256, BN = (tile == 256) ? 256 : (tile == 320) ? 192 : 128;
     const int ktiles = (int)(((long)K * (i8 ? 1 : 2)) >> 7);
     return kmi_pick_splits(M, N, K, BM, BN, ktiles, ws);
 }

@@ -73,7 +73,7 @@ __device__ __forceinline__ void store_partial(const GemmArgs& p, acc_t (&acc)[FM
                     u4_t v;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const auto elem = acc_elem<(FM * FN >= 16)>(acc[i][j][4 * g + r]);   // a scalar copy:
+                        const auto elem = acc_elem<(FM * FN >= 12)>(acc[i][j][4 * g + r]);   // a scalar copy:
                         v[r] = __builtin_bit_cast(uint32_t, elem);       // bit_cast needs an addressable scalar
                     }
                     *reinterpret_cast<u4_t*>(dst + (long)m * N + n) = v;
@@ -159,7 +159,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         }
     } else {
         constexpr int WN = BN / 2;                       // columns per wave
-        constexpr bool BIG = FM * FN >= 16;              // accumulators in AGPRs, read explicitly
+        constexpr bool BIG = FM * FN >= 12;              // accumulators in AGPRs, read explicitly
         constexpr int PITCH = WN * 2 + 8;                // bytes
         constexpr int CPR = WN * 2 / 16;                 // 16-byte chunks per row
         char* patch = smem + wave * (32 * PITCH);
@@ -253,6 +253,23 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
             for (int k = 0; k < NK; ++k) {                   // all reads first: one LDS round trip, not NK
                 const int idx = k * 64 + lane;
                 v[k] = *reinterpret_cast<const u4_t*>(patch + (idx / CPR) * PITCH + (idx % CPR) * 16);
+            }
+            if constexpr (64 % CPR != 0) {                   // 96 columns per wave: the column changes with k
+                static_assert((32 * CPR) % 64 == 0, "whole 16-byte chunks per lane");
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int idx = k * 64 + lane;
+                    const int m = mw + i * 32 + idx / CPR, n = nw + (idx % CPR) * 8;
+                    half_t* d = outp + (long)m * N + n;
+                    if (wide) {
+                        if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(d));
+                    } else {
+                        if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
+                        if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                continue;
             }
             const int n = nw + (lane % CPR) * 8;             // CPR divides 64: the column is the same for every k
             half_t* dst = outp + (long)(mw + i * 32 + lane / CPR) * N + n;

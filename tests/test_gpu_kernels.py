@@ -346,13 +346,13 @@ def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
     assert torch.equal(acc, again) and torch.equal(acc, ops.w8a8_gemm_acc_i32(a8, w8, N))
 
 
-@pytest.mark.parametrize("K", [128, 384])
-def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K):
+@pytest.mark.parametrize("K,N,wide", [(128, 7808, 256), (384, 7808, 256), (384, 7680, 320), (128, 7808, 320)])
+def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K, N, wide):
     """More 256 x 256 tiles than compute units (9 x 31 = 279, ragged in M and N): the tiled-weight W8A8 and fp16 GEMMs
     then run one workgroup per CU that walks the tiles and starts a tile's first loads while the previous one is
     written out.  K = 128 is shorter than the load pipeline.  Outputs equal the 128-row-tile kernel's bit for bit
     (same accumulation order) and the oracle's on sampled rows, with and without a bias."""
-    M, N = 2100, 7808
+    M = 2100                                                # N = 7680: 9 x 40 tiles of 256 x 192, tiles that start in the middle of a weight strip
     p = prep(N, K, seed=K)
     x = O.synth_acts(M, K, seed=K + 1)
     a8_np, sx_np = O.quant_act_i8(x)
@@ -366,7 +366,7 @@ def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K):
     ops.dequant_interleaved_int4_to_fp16(w16_t, dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), 128, tiled=True)
     a8, sx, xd, bias, s1 = dev(a8_np), dev(sx_np), dev(x), dev(bias_np), dev(p["scales_1"])
     got = {}
-    for tile in (256, 128):
+    for tile in (wide, 128):
         ops.force_gemm_tile(tile)
         ops.force_gemm_splits(1)
         try:
@@ -379,11 +379,11 @@ def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K):
         finally:
             ops.force_gemm_tile(0)
             ops.force_gemm_splits(0)
-    for a, b in zip(got[256], got[128]):
+    for a, b in zip(got[wide], got[128]):
         assert torch.equal(a, b)
-    assert_same_bits(host(got[256][0])[rows], ref8)
-    assert_same_bits(host(got[256][1])[rows], ref8_b)
-    assert O.max_abs_rel(host(got[256][2])[rows], O.gemm_f16(x[rows], p["w16"])) < 2e-3
+    assert_same_bits(host(got[wide][0])[rows], ref8)
+    assert_same_bits(host(got[wide][1])[rows], ref8_b)
+    assert O.max_abs_rel(host(got[wide][2])[rows], O.gemm_f16(x[rows], p["w16"])) < 2e-3
 
 
 @pytest.mark.parametrize("tile", [64, 128, 256])
@@ -409,7 +409,7 @@ def test_gemm_w4a16_f16_w8a16(ops, M, tile):
     assert O.max_abs_rel(host(out816), O.gemm_w8a16(x, p["w8"], p["scales_1"])) < 2e-3
 
 
-@pytest.mark.parametrize("tile", [64, 128, 192, 256])
+@pytest.mark.parametrize("tile", [64, 128, 192, 256, 320])     # 320: 256 x 192 tiles (tiled operands; row-major runs 256 x 256)
 def test_gemm_tiled_operands_match_row_major(ops, tile):
     N, K, M = 384, 1024, 150
     p = prep(N, K)
