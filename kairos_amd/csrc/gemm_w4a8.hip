@@ -446,7 +446,7 @@ static int w4a8_head_cols(int M, int N) {
 
 static int w4a8_tile(int M, int N, int K) {
     const int forced = kmi_forced_tile();
-    if (forced == 128 || forced == 192 || forced == 256) return forced;
+    if (forced == 128 || forced == 192 || forced == 256 || forced == 512) return forced;
     if (forced == 130) return (K % 256 == 0) ? 130 : 128;    // 128 x 128 tile, two wave quartets per workgroup
     if (forced == 448) return w4a8_head_cols(M, N) > 0 ? 448 : 256;
     const Workspace roomy{reinterpret_cast<void*>(16), (size_t)64 << 20};
@@ -482,12 +482,17 @@ static int w4a8_tile(int M, int N, int K) {
         const long tail = (long)(TN - head) * TM * 2;
         c448 = 2.0 * fixed + ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256;
     }
-    if (c128 <= c192 && c128 <= c256 && c128 <= c448) {
+    if (c128 <= c192 && c128 <= c256 && c128 <= c448 && (M < 512 || c128 <= cost(512, 128, 0.93, 0.93, 256))) {
         // At most one workgroup per CU: two wave quartets per workgroup, each on half of the workgroup's K range
         // (28672 columns M=128: 28.0 against 32.5 us; 6144 columns M=512: 24.8 against 29.6; 4096 x 14336 M=256 with
         // four splits: 33.1 against 35.5; level elsewhere).  More workgroups than CUs overlap each other already.
         return two_quartets ? 130 : 128;
     }
+    // 512 x 128: the accumulators of a 256 x 256 tile, but one decoded weight serves 512 activation rows, i.e. half the
+    // decode instructions per MFMA (28672 columns M=1024: 124.5 against 134.2 us; M=4096: 460 against 472; 6144 columns
+    // M=2048: 56.6 against 59.8).  Not below 512 rows, where half of the tile would be padding.
+    const double c512 = M >= 512 ? cost(512, 128, 0.93, 0.93, 256) : 1e30;
+    if (c512 < c448 && c512 < c192 && c512 < c256) return 512;
     if (c448 <= c192 && c448 <= c256) return 448;
     return c192 <= c256 ? 192 : 256;
 }
@@ -513,7 +518,8 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
     } else {
         rc = tile == 256 ? launch_w4a8<KIND, 256, 256>(a, ws, st)
            : tile == 192 ? launch_w4a8<KIND, 256, 128>(a, ws, st)
-           : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
+           : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st)
+           : tile == 512 ? launch_w4a8<KIND, 512, 128>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
     }
     if (rc != KMI_OK) return rc;
     return kmi_check_launch(fn);

@@ -277,7 +277,8 @@ def test_conversion_qwen_shapes_against_oracle(ops, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(4096, 28672, 4096), (2048, 4096, 14336), (1024, 6144, 4096), (512, 28672, 4096),
                                    (256, 4096, 4096), (2048, 28672, 4096), (4096, 6144, 4096),    # these two: two launches
-                                   (128, 28672, 4096), (1024, 4096, 14336), (128, 4096, 14336)])  # two wave quartets per workgroup
+                                   (128, 28672, 4096), (1024, 4096, 14336), (128, 4096, 14336),   # two wave quartets per workgroup
+                                   (1024, 28672, 4096), (4096, 4096, 14336)])                      # 512 x 128 tiles
 def test_w4a8_lane_full_size(ops, M, N, K):
     """The W4A8 lane at the benchmark's sizes.  (a) On the exactly computable inputs of the W8A8 full-size test (tables
     s = 1, z = -8, sparse +-127 activations, channel scale 1/128) the whole fp16 output is one known rounding of an

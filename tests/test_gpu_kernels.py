@@ -287,7 +287,7 @@ def test_gemm_w8a8_path(ops, M, tile):
     assert_same_bits(host(out), ref)
 
 
-@pytest.mark.parametrize("tile", [0, 128, 130, 192, 256])       # 130: the 128 x 128 tile with two wave quartets
+@pytest.mark.parametrize("tile", [0, 128, 130, 192, 256, 512])  # 130: the 128 x 128 tile with two wave quartets; 512: 512 x 128
 @pytest.mark.parametrize("M", GEMM_M)
 def test_gemm_w4a8_bit_exact(ops, M, tile):
     """W4A8 (int4 weights decoded to the converter's int8 values inside the int8 MFMA GEMM): int32 accumulators and
@@ -316,7 +316,7 @@ def test_gemm_w4a8_bit_exact(ops, M, tile):
     assert_same_bits(host(out_b), out_b_ref)
 
 
-@pytest.mark.parametrize("tile,splits", [(128, 1), (256, 1), (128, 3), (256, 2), (192, 1), (192, 4), (130, 1), (130, 2), (130, 3), (0, 0)])
+@pytest.mark.parametrize("tile,splits", [(128, 1), (256, 1), (128, 3), (256, 2), (192, 1), (192, 4), (130, 1), (130, 2), (130, 3), (512, 1), (512, 2), (0, 0)])
 def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
     """Arbitrary tables (every table byte differs from row to row and group to group, values beyond the int8 range are
     clipped as the converter clips them), full-range activations, K split over workgroups: accumulators equal the
