@@ -288,6 +288,15 @@ __device__ __forceinline__ h8_t dequant_nibble_r(const u4_t& u, h2_t s2, h2_t z2
     return o;
 }
 
+// f(integral_constant<int, B>) ... f(integral_constant<int, E - 1>), unrolled at compile time
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 // =================================================================================================
 // W4A16 for M up to a few hundred rows: wave-private weights.
 //
@@ -295,12 +304,13 @@ __device__ __forceinline__ h8_t dequant_nibble_r(const u4_t& u, h2_t s2, h2_t z2
 // memory: every weight passes through LDS (a write and two fragment reads) and one wave per SIMD
 // serialises decode, LDS and load issue.  Here a workgroup tile is BM rows x 128 columns and each
 // wave owns 32 of the columns for itself, so its weights never touch LDS: lane (n = lane%32,
-// h = lane/32) loads the 16-byte chunk h of row n of the 64-wide k-tile (32 weights), decodes its four
-// 8-weight planes exactly as the converters do, and trades two of them with lane n of the other half
-// (v_permlane32_swap) so that each half holds the k-blocks its MFMA operand position needs:
-//   lower lanes  k 0-7, 32-39, 16-23, 48-55      upper lanes  k 8-15, 40-47, 24-31, 56-63
-// i.e. MFMA j of the four per k-tile covers the 16-wide k-step {0, 2, 1, 3}[j]; the activation fragment
-// of that k-step is read from LDS.  Only the activations are staged (direct-to-LDS loads, PF+1 stages),
+// h = lane/32) loads the 16-byte chunk h of row n of the 64-wide k-tile (32 weights) and decodes its four
+// 8-weight planes exactly as the converters do; plane p is k 32h + 8p .. + 7 of the k-tile.  Which sixteen k
+// an MFMA sums is free as long as both operands agree, so MFMA p of the four per k-tile takes plane p as it
+// lies -- k 8p..8p+7 in the lower half-wave, 32+8p..32+8p+7 in the upper -- and the activation fragment is
+// read from LDS at those k (chunk 4h + p of the row): no lane of the wave ever hands a weight to another
+// (a v_permlane32_swap costs 13-16 cycles of the vector ALU, three ordinary instructions; sixteen of them per
+// k-tile were 40 % of the decode).  Only the activations are staged (direct-to-LDS loads, PF+1 stages),
 // shared by the four column waves.  The workgroup has KH such wave quartets; quartet q takes k-tiles
 // q, q+KH, ... and the quartets' accumulators meet in LDS at the end (fixed order).  A scale and a
 // scaled zero arrive in ONE load (lower lanes fetch the scale, upper lanes the zero of the same column)
@@ -376,41 +386,28 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
     // landed -- its weights and scales for the decode, its activations for the fragment reads issued during
     // k-step 3 -- while the PF-2 younger k-tiles may stay in flight (OPS instructions each, issued in whole
     // groups); the barrier also frees the LDS stage of k-tile j-1 for the loads of k-tile j+PF.
-#define KMI_WP_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
     auto tile_barrier = [&](auto keep_tiles) {
         constexpr int KEEP = decltype(keep_tiles)::value * OPS;
-        static_assert(KEEP == 6 || KEEP == 8 || KEEP == 9 || KEEP == 12 || KEEP == 18, "no immediate for this depth");
-        if constexpr (KEEP == 6) KMI_WP_BARRIER(6);
-        else if constexpr (KEEP == 8) KMI_WP_BARRIER(8);
-        else if constexpr (KEEP == 9) KMI_WP_BARRIER(9);
-        else if constexpr (KEEP == 12) KMI_WP_BARRIER(12);
-        else KMI_WP_BARRIER(18);
+        static_assert(KEEP >= 0 && KEEP < 64, "vmcnt is a six-bit count");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(KEEP) : "memory");
     };
 
     const int fr = lane & 31;
     const NibConsts nc = nib_consts();
     u4_t pl[2][4];                                   // decoded weights: [parity of the k-tile][MFMA of the k-tile]
     u4_t fa[2][FM];                                  // activation fragments: [parity of the k-step]
-    // pl[.][jj] covers k-step {0, 2, 1, 3}[jj]
+    // pl[.][jj] is plane jj of the lane's own chunk: k 32*hl + 8*jj .. + 7; the activations of the same k
     auto read_frags = [&](int j, int jj, int set) {
-        const int ks = (jj == 1) ? 2 : (jj == 2) ? 1 : jj;
         const char* st = ring + (j % NSA) * A_STAGE;
 #pragma unroll
-        for (int i = 0; i < FM; ++i) fa[set][i] = *reinterpret_cast<const u4_t*>(st + lds_off(i * 32 + fr, 2 * ks + hl));
+        for (int i = 0; i < FM; ++i) fa[set][i] = *reinterpret_cast<const u4_t*>(st + lds_off(i * 32 + fr, 4 * hl + jj));
     };
-    // planes 2*half, 2*half+1 of k-tile set S -> pl[par][2*half .. 2*half+1]; lower lanes keep the even plane of
-    // both chunks, upper lanes the odd one
+    // planes 2*half, 2*half+1 of k-tile set S -> pl[par][2*half .. 2*half+1]
     auto decode_half = [&](auto set, auto half, int par, h2_t s2, h2_t z2) {
         constexpr int S = decltype(set)::value, H = decltype(half)::value;
         const u4_t raw = rb[S];
-        const u4_t e = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H>(raw, s2, z2, nc));
-        const u4_t o = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H + 1>(raw, s2, z2, nc));
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const auto x = __builtin_amdgcn_permlane32_swap(e[w], o[w], false, false);
-            pl[par][2 * H][w] = x[0];
-            pl[par][2 * H + 1][w] = x[1];
-        }
+        pl[par][2 * H] = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H>(raw, s2, z2, nc));
+        pl[par][2 * H + 1] = __builtin_bit_cast(u4_t, dequant_nibble_r<2 * H + 1>(raw, s2, z2, nc));
     };
     auto scales_of = [&](auto set, h2_t& s2, h2_t& z2) {
         constexpr int S = decltype(set)::value;
@@ -449,13 +446,13 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         read_frags(j, 1, 1);
         mfma_block(par, 0, 0);
         decode_half(SetN{}, I0{}, par ^ 1, s2, z2);
-        interleave(std::integral_constant<int, 36>{}, std::integral_constant<int, FM>{}, I0{});
+        interleave(std::integral_constant<int, 28>{}, std::integral_constant<int, FM>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
         // k-step 1 under the second half
         read_frags(j, 2, 0);
         mfma_block(par, 1, 1);
         decode_half(SetN{}, I1{}, par ^ 1, s2, z2);
-        interleave(std::integral_constant<int, 44>{}, std::integral_constant<int, FM>{}, I0{});
+        interleave(std::integral_constant<int, 36>{}, std::integral_constant<int, FM>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
         // k-step 2 under the loads of k-tile j+PF (their registers and their LDS stage are free now)
         read_frags(j, 3, 1);
@@ -470,16 +467,9 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // ---- pipeline: PF k-tiles in flight per wave
-    {
-        int j = 0;
-        auto prime = [&](auto set) { issue(set, j); ++j; __builtin_amdgcn_sched_barrier(0); };
-        prime(std::integral_constant<int, 0>{});
-        if constexpr (PF > 1) prime(std::integral_constant<int, 1>{});
-        if constexpr (PF > 2) prime(std::integral_constant<int, 2>{});
-        if constexpr (PF > 3) prime(std::integral_constant<int, 3>{});
-        static_assert(PF == 4, "the loop below is unrolled for four register sets");
-    }
+    // ---- pipeline: PF k-tiles in flight per wave (register set = k-tile index modulo PF, a compile-time constant)
+    static_assert(PF % 2 == 0 && PF >= 4, "the parity of a k-tile must follow from its register set");
+    static_for<0, PF>([&](auto set) { issue(set, decltype(set)::value); __builtin_amdgcn_sched_barrier(0); });
     {   // k-tile 0: decoded in the open
         tile_barrier(std::integral_constant<int, PF - 1>{});
         h2_t s2, z2;
@@ -490,17 +480,11 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
         __builtin_amdgcn_sched_barrier(0);
     }
     int j = 0;
-    for (; j + PF <= T; j += PF) {
-        body(std::integral_constant<int, 0>{}, j);
-        body(std::integral_constant<int, 1>{}, j + 1);
-        body(std::integral_constant<int, 2>{}, j + 2);
-        body(std::integral_constant<int, 3>{}, j + 3);
-    }
-    if (j < T) { body(std::integral_constant<int, 0>{}, j); ++j; }
-    if (j < T) { body(std::integral_constant<int, 1>{}, j); ++j; }
-    if (j < T) { body(std::integral_constant<int, 2>{}, j); ++j; }
+    for (; j + PF <= T; j += PF) static_for<0, PF>([&](auto set) { body(set, j + decltype(set)::value); });
+    static_for<0, PF - 1>([&](auto set) {
+        if (j < T) { body(set, j); ++j; }
+    });
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // no load outlives its stage
-#undef KMI_WP_BARRIER
 
     // ---- the quartets' partial sums meet in LDS, added to quartet 0 in quartet order
     if constexpr (KH > 1) {
@@ -899,8 +883,9 @@ static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st
 template <int BM, int KH = 2>
 static int launch_w4a16_wp(const GemmArgs& a_in, const Workspace& ws, hipStream_t st) {
     GemmArgs a = a_in;
-    constexpr int PF = 4;
+    constexpr int PF = 4;                                        // k-tiles in flight per wave (8 measured 3-5 % slower at 32 / 64 rows)
     constexpr size_t lds = (size_t)KH * (PF + 1) * BM * 128;
+    static_assert(lds <= 160 * 1024, "the activation ring must fit the LDS of a CU");
     void (*fn)(GemmArgs) = gemm_w4a16_wp_kernel<BM, KH, PF>;
     static thread_local bool raised = false;
     if (lds > 64 * 1024 && !raised) {

@@ -91,27 +91,38 @@ __device__ __forceinline__ void static_for(F&& f) {
 // the other's MFMAs -- what two workgroups per CU do for each other, without a second output tile or partial sums in
 // memory.  Their int32 accumulators meet in LDS at the end (integers: the order does not matter).  Small tiles only:
 // two waves per SIMD leave 256 registers each.
-template <int KIND, int BM, int BN, int KH = 1>
-__global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
+//
+// MW = 2: two wave quartets on ONE pipeline.  Quartet h multiplies rows h*BM/2 .. of the tile against all BN columns;
+// both read the same LDS stages and all eight waves bring the activation rows in, but only quartet 0 loads, decodes
+// and stores the weights.  With one wave per SIMD every instruction of the stage -- some 200 against 32 MFMAs --
+// queues on that wave's own issue port (one instruction per four cycles), which the MFMAs cannot cover; the second
+// wave of the SIMD issues its MFMAs and fragment reads into those gaps.
+template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
+__global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     static_assert(KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC, "int8 accumulation");
     constexpr int NS = 4;
-    constexpr int FM = BM / 64, FN = BN / 64;
+    static_assert(MW == 1 || (MW == 2 && KH == 1), "two quartets share either the K range or the tile's rows");
+    constexpr int BMW = BM / MW;                            // tile rows of one quartet
+    constexpr int FM = BMW / 64, FN = BN / 64;
     constexpr int ROWS = BM + BN;
     constexpr int STAGE = ROWS * 64;
-    constexpr int NLA = BM * 4 / 256;                       // direct activation loads per thread and stage
+    constexpr int NLA = BM * 4 / (256 * MW);                // direct activation loads per thread and stage
     constexpr int NLA0 = (NLA + 1) / 2, NLA1 = NLA - NLA0;  // issued behind the barrier / in front of it
     constexpr int CPT = BN * 2 / 256;                       // packed 16-byte chunks per thread and stage
     static_assert(BM % 64 == 0 && (BN == 128 || BN == 256) && NLA >= 2, "tile shapes this staging scheme covers");
     using acc_t = i16_t;
 
-    static_assert(KH == 1 || (KH == 2 && FM * FN < 16), "two quartets: accumulators in VGPRs, 256 registers per wave");
+    static_assert(KH * MW == 1 || FM * FN < 16, "two quartets: 256 registers per wave");
     extern __shared__ __attribute__((aligned(16))) char smem_all[];
 
     const int tid = threadIdx.x & 255;                       // index inside the quartet
-    const int kq = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    char* const smem = smem_all + kq * (NS * STAGE);         // this quartet's ring
+    const int quartet = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    const int kq = MW == 1 ? quartet : 0;                    // KH = 2: which half of the K range
+    const int mh = MW == 2 ? quartet : 0;                    // MW = 2: which half of the tile's rows
+    char* const smem = smem_all + kq * (NS * STAGE);         // this quartet's ring (MW = 2: the one ring)
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_all = mh * 4 + wave;                      // among the waves that share the ring
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
@@ -133,11 +144,11 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-    // ---- activation side: load i of wave w fills the KiB region R = 4*i + w = tile rows 16R .. 16R+15
+    // ---- activation side: load i of wave w fills the KiB region R = 4*MW*i + w = tile rows 16R .. 16R+15
     uint32_t voff_a[NLA];
 #pragma unroll
     for (int i = 0; i < NLA; ++i) {
-        const int row = 16 * (4 * i + wave) + (lane >> 2);
+        const int row = 16 * (4 * MW * i + wave_all) + (lane >> 2);
         const int c = (lane & 3) ^ ((row >> 2) & 3);
         int m = m0 + row;
         m = m < M ? m : M - 1;
@@ -164,12 +175,12 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
 
     auto clamp_stage = [&](int u) { return t0 + (u < T ? u : T - 1); };   // past the end: harmless reloads
     auto issue_a_half = [&](int u, int slot, int h) {        // h = 0: loads 0 .. NLA0-1, h = 1: the rest
-        char* dst = smem + slot * STAGE + wave * 1024;
+        char* dst = smem + slot * STAGE + wave_all * 1024;
         const uint32_t sa = (uint32_t)clamp_stage(u) * 64u;
 #pragma unroll
         for (int i = 0; i < NLA; ++i) {
             if ((i < NLA0) != (h == 0)) continue;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, voff_a[i], sa, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * (4096 * MW)), 16, voff_a[i], sa, 0, 0);
         }
     };
     auto issue_raw = [&](int u, auto sp, auto gp) {
@@ -240,7 +251,7 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
     int off_a[2], off_b[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-        off_a[s] = (wm * (BM / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
+        off_a[s] = (mh * BMW + wm * (BMW / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
         off_b[s] = (BM + wn * (BN / 2) + fr) * 64 + (((2 * s + fkh) ^ fsw) << 4);
     }
     u4_t fa[2][FM], fb[2][FN];
@@ -258,23 +269,34 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
     // ---- prologue.  Issue order mirrors the loop's, so that the loop's wait counts hold from iteration 0 on:
     //   [A0, packed 0, packed 1, scale/zero of group 0] [A1] [A2 first half, packed 2, scale/zero of group 1]
     //   [A2 second half] [A3 first half, packed 3]
+    // DEC: this wave stages weights (always, except the second quartet of MW = 2); the others issue the same
+    // barriers and only the activation loads, so their wait counts leave the weight-side loads out.
+    auto pipeline = [&](auto dec_) {
+    constexpr bool DEC = decltype(dec_)::value;
+    constexpr int CPE = DEC ? CPT : 0, SZ = DEC ? 2 : 0;     // weight-side loads of this wave: packed chunks, scale + zero
     issue_a_half(0, 0, 0); issue_a_half(0, 0, 1);
-    issue_raw(0, I0{}, I0{});
-    issue_raw(1, I1{}, I0{});
-    issue_sz(0, I0{});
+    if constexpr (DEC) {
+        issue_raw(0, I0{}, I0{});
+        issue_raw(1, I1{}, I0{});
+        issue_sz(0, I0{});
+    }
     __builtin_amdgcn_sched_barrier(0);
     issue_a_half(1, 1, 0); issue_a_half(1, 1, 1);
     issue_a_half(2, 2, 0);
-    issue_raw(2, I0{}, I1{});
-    issue_sz(2, I1{});
+    if constexpr (DEC) {
+        issue_raw(2, I0{}, I1{});
+        issue_sz(2, I1{});
+    }
     __builtin_amdgcn_sched_barrier(0);
     issue_a_half(2, 2, 1);
     issue_a_half(3, 3, 0);
-    issue_raw(3, I1{}, I1{});
+    if constexpr (DEC) issue_raw(3, I1{}, I1{});
     __builtin_amdgcn_sched_barrier(0);
-    wait_vmcnt<NLA + (NLA0 + CPT + 2) + NLA1 + (NLA0 + CPT)>();
-    static_for<0, 4 + 9 * CPT>([&](auto it) { work_item(I0{}, I0{}, I1{}, it, 0); });       // stage 0 (builds the table)
-    static_for<0, 9 * CPT>([&](auto it) { work_item(I1{}, I0{}, I0{}, it, 1); });           // stage 1
+    wait_vmcnt<NLA + (NLA0 + CPE + SZ) + NLA1 + (NLA0 + CPE)>();
+    if constexpr (DEC) {
+        static_for<0, 4 + 9 * CPT>([&](auto it) { work_item(I0{}, I0{}, I1{}, it, 0); });       // stage 0 (builds the table)
+        static_for<0, 9 * CPT>([&](auto it) { work_item(I1{}, I0{}, I0{}, it, 1); });           // stage 1
+    }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     read_frags(0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
@@ -289,16 +311,16 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
         constexpr int SLOT = 2 * GP + SP;                    // t % 4
         using GN = std::integral_constant<int, GP ^ 1>;      // group parity of stage t+2
         using WT = std::integral_constant<int, SP == 0 ? 1 : 0>;   // stage t+2 opens a group: build its table first
-        constexpr int NTAB = SP == 0 ? 4 : 0, NITEMS = NTAB + 9 * CPT;
+        constexpr int NTAB = SP == 0 ? 4 : 0, NITEMS = DEC ? NTAB + 9 * CPT : 0;
         constexpr int COST = 2 * NTAB + 9 * CPT;            // a table word costs about two lookups
         constexpr int NSLOTS = 2 * NMF;
-        constexpr int NP1 = NLA1, NP2 = NLA0 + CPT + (SP == 0 ? 2 : 0);   // loads in front of / behind the barrier
+        constexpr int NP1 = NLA1, NP2 = NLA0 + CPE + (SP == 0 ? SZ : 0);  // loads in front of / behind the barrier
         constexpr int RD_SLOTS = NMF >= 8 ? NMF / 2 : NMF;   // fragment reads go to the first slots of a block,
         constexpr int LD_FROM = NMF >= 8 ? NMF / 2 : 0;      // loads to the last ones (small tiles: everywhere)
         // everything issued up to two iterations ago has landed: activations of stage t+1, the packed chunks of
         // stage t+2 and, on even t, scale and zero of its group.  Younger: second half of A(t+2), [first half of
         // A(t+3), packed t+3, and on odd t the scale/zero pair issued by the even iteration before].
-        wait_vmcnt<NLA1 + NLA0 + CPT + (SP == 1 ? 2 : 0)>();
+        wait_vmcnt<NLA1 + NLA0 + CPE + (SP == 1 ? SZ : 0)>();
         const uint32_t sa3 = (uint32_t)clamp_stage(t + 3) * 64u, sa4 = (uint32_t)clamp_stage(t + 4) * 64u;
         const uint32_t sb4 = (uint32_t)clamp_stage(t + 4) * 128u;
         const uint32_t so4 = (uint32_t)(clamp_stage(t + 4) >> 1) * (uint32_t)N * 2u;
@@ -322,11 +344,11 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
             static_for<l0, l1>([&](auto l_) {
                 constexpr int l = decltype(l_)::value;
                 if constexpr (BLK == 0) {                    // second half of the activation rows of stage t+3
-                    char* dst = smem + ((SLOT + 3) & 3) * STAGE + wave * 1024;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + (NLA0 + l) * 4096), 16, voff_a[NLA0 + l], sa3, 0, 0);
+                    char* dst = smem + ((SLOT + 3) & 3) * STAGE + wave_all * 1024;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + (NLA0 + l) * (4096 * MW)), 16, voff_a[NLA0 + l], sa3, 0, 0);
                 } else if constexpr (l < NLA0) {             // first half of the activation rows of stage t+4
-                    char* dst = smem + SLOT * STAGE + wave * 1024;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + l * 4096), 16, voff_a[l], sa4, 0, 0);
+                    char* dst = smem + SLOT * STAGE + wave_all * 1024;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + l * (4096 * MW)), 16, voff_a[l], sa4, 0, 0);
                 } else if constexpr (l < NLA0 + CPT) {       // packed chunks of stage t+4
                     raw[SP][GP][l - NLA0] = __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b + 16u * (l - NLA0), sb4, 0));
                 } else if constexpr (l == NLA0 + CPT) {      // scale / scaled zero of the group stage t+4 opens
@@ -361,6 +383,13 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
         iteration(I0{}, I0{}, t);
         iteration(I1{}, I0{}, t + 1);
     }
+    };
+    if constexpr (MW == 1) {
+        pipeline(std::true_type{});
+    } else {
+        if (mh == 0) pipeline(std::true_type{});
+        else pipeline(std::false_type{});
+    }
     // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
@@ -385,21 +414,25 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a8_kernel(GemmArgs p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] += red[((i * FN + j) * 16 + e) * 256 + tid];
     }
-    if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, split, m0, n0, wave, lane);
-    else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, m0, n0, wave, lane);
-    else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, m0, n0, wave, lane);
+    // each quartet of MW = 2 writes its half of the tile's rows out, with patches of its own
+    constexpr int EPI_LDS = 4 * 32 * ((BN / 2) * 2 + 8);
+    char* const epi = smem + mh * EPI_LDS;
+    const int me = m0 + mh * BMW;
+    if (p.splits > 1) store_partial<BMW, BN, FM, FN>(p, acc, split, me, n0, wave, lane);
+    else if (p.bias) gemm_epilogue<KIND, BMW, BN, true, FM, FN>(p, acc, epi, me, n0, wave, lane);
+    else gemm_epilogue<KIND, BMW, BN, false, FM, FN>(p, acc, epi, me, n0, wave, lane);
 #endif
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-template <int KIND, int BM, int BN, int KH = 1>
+template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
 static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const Workspace ws = (a.n_begin == 0 && a.n_cols == a.N) ? ws_in : Workspace{nullptr, 0};   // column ranges: no split over K
     constexpr size_t lds = (size_t)KH * 4 * (BM + BN) * 64;
-    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN, KH>;
+    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN, KH, MW>;
     static thread_local bool raised = false;                 // per instantiation, per thread
     if (lds > 64 * 1024 && !raised) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -417,7 +450,7 @@ static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t
     if (KH == 2 && (stages % UNIT != 0)) return kmi_set_error(KMI_E_SHAPE, "gemm_w4a8: two quartets need K %% 256 == 0 (K=%d)", a.K);
     a.splits = s < 2 ? 1 : s;
     a.partial = a.splits > 1 ? ws.ptr : nullptr;
-    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256 * KH);
+    const dim3 grid(((a.n_cols + BN - 1) / BN) * ((a.M + BM - 1) / BM) * a.splits), block(256 * KH * MW);
     hipLaunchKernelGGL(fn, grid, block, lds, st, a);
     if (a.splits > 1) {
         const long quads = (long)a.M * a.N / 4;
@@ -428,7 +461,7 @@ static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t
 
 // Tile choice by a small cost model fitted to MI355X timings (microseconds).  A 256 x 256 tile over K = 4096 takes
 // about 69.5 us with one workgroup per CU (0.40 of the int8 peak with the decode between the MFMAs); a 256 x 128 tile
-// (selector 192) 0.59 of that, a 128 x 128 tile 0.50 alone on a CU and 0.67 per pair when two share one (its decode
+// (selector 192) 0.59 of that (0.54 while every workgroup has a CU to itself), a 128 x 128 tile 0.50 alone on a CU and 0.67 per pair when two share one (its decode
 // makes it VALU-bound).  Workgroups run in rounds over the CUs; a split over K divides the tile time and adds the
 // partial-sum traffic and the reduce kernel.  Checked against sweeps of the Llama-3-8B shapes, M = 128 .. 4096:
 // 6144 columns M = 1024 -> 256 x 128 (41.7 us against 48.8 with 128 x 128 and 58.4 with 256 x 256), 28672 columns
@@ -467,7 +500,7 @@ static int w4a8_tile(int M, int N, int K) {
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     const int s128 = kmi_pick_splits(M, N, K, 128, 128, K >> 7, roomy);
     const bool two_quartets = (K % 256 == 0) && tiles128 * s128 <= 256;
-    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.59, 0.59, 256);
+    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.54, 0.59, 256);
     double c128 = cost(128, 128, 0.45, 0.67, 512);
     if (two_quartets) {
         const double w = (double)(tiles128 * s128);
@@ -482,16 +515,17 @@ static int w4a8_tile(int M, int N, int K) {
         const long tail = (long)(TN - head) * TM * 2;
         c448 = 2.0 * fixed + ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256;
     }
-    if (c128 <= c192 && c128 <= c256 && c128 <= c448 && (M < 512 || c128 <= cost(512, 128, 0.93, 0.93, 256))) {
+    if (c128 <= c192 && c128 <= c256 && c128 <= c448 && (M < 512 || c128 <= cost(512, 128, 0.90, 0.90, 256))) {
         // At most one workgroup per CU: two wave quartets per workgroup, each on half of the workgroup's K range
         // (28672 columns M=128: 28.0 against 32.5 us; 6144 columns M=512: 24.8 against 29.6; 4096 x 14336 M=256 with
         // four splits: 33.1 against 35.5; level elsewhere).  More workgroups than CUs overlap each other already.
         return two_quartets ? 130 : 128;
     }
-    // 512 x 128: the accumulators of a 256 x 256 tile, but one decoded weight serves 512 activation rows, i.e. half the
-    // decode instructions per MFMA (28672 columns M=1024: 124.5 against 134.2 us; M=4096: 460 against 472; 6144 columns
-    // M=2048: 56.6 against 59.8).  Not below 512 rows, where half of the tile would be padding.
-    const double c512 = M >= 512 ? cost(512, 128, 0.93, 0.93, 256) : 1e30;
+    // 512 x 128 on eight waves (two quartets, 256 rows each): as many accumulators per SIMD as a 256 x 256 tile, but one
+    // decoded weight serves 512 activation rows, i.e. half the decode instructions per MFMA (28672 columns M=1024: 123.7
+    // against 134.7 us; M=4096: 471 against 488; 6144 columns M=2048: 55.8 against 61.9; four waves of 256 x 64 each on
+    // the same tile: 127.5 / 475 / 58.3).  Not below 512 rows, where half of the tile would be padding.
+    const double c512 = M >= 512 ? cost(512, 128, 0.90, 0.90, 256) : 1e30;
     if (c512 < c448 && c512 < c192 && c512 < c256) return 512;
     if (c448 <= c192 && c448 <= c256) return 448;
     return c192 <= c256 ? 192 : 256;
@@ -519,7 +553,7 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
         rc = tile == 256 ? launch_w4a8<KIND, 256, 256>(a, ws, st)
            : tile == 192 ? launch_w4a8<KIND, 256, 128>(a, ws, st)
            : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st)
-           : tile == 512 ? launch_w4a8<KIND, 512, 128>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
+           : tile == 512 ? launch_w4a8<KIND, 512, 128, 1, 2>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
     }
     if (rc != KMI_OK) return rc;
     return kmi_check_launch(fn);
