@@ -116,6 +116,21 @@ def compress_segments(perf_list):
     return seg
 
 
+def choose_lane(times, prev_comp='', stickiness=0.01, prefer_resident=0.04):
+    """The lane for one M from the measured times {lane: t}: the fastest; unless a lane that reads only the resident
+    int4 weight (names starting with 'w4') is within `prefer_resident` of it; unless the previous M's lane is within
+    `stickiness` of that choice.  -> (lane, its time)."""
+    best_t, best_comp = min((t, c) for c, t in times.items())
+    resident = [(t, c) for c, t in times.items() if c.startswith('w4')]
+    if prefer_resident > 0 and resident and not best_comp.startswith('w4'):
+        t4, c4 = min(resident)
+        if t4 <= best_t * (1.0 + prefer_resident):
+            best_t, best_comp = t4, c4
+    if prev_comp in times and times[prev_comp] <= best_t * (1.0 + stickiness):
+        best_t, best_comp = times[prev_comp], prev_comp
+    return best_comp, best_t
+
+
 def lane_allowed(comp_type, m):
     if 'gemv' in comp_type and m > GEMV_MAX_M:
         return False
@@ -166,7 +181,6 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
     prev_comp = ''
     for m in input_len:
         x = torch.randn((1, m, K), dtype=torch.float16, device='cuda')
-        best_t, best_comp = float('inf'), ''
         orig_t = float('inf')
         times = {}
         for comp in comp_type_list:
@@ -187,17 +201,9 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
             if details is not None:
                 details.append({"shape": [N, K], "m": m, "comp": comp, "ms": t})
             times[comp] = t
-            if t < best_t:
-                best_t, best_comp = t, comp
             if 'w4' in comp and t < orig_t:
                 orig_t = t
-        resident = [(t, c) for c, t in times.items() if c.startswith('w4')]
-        if prefer_resident > 0 and resident and not best_comp.startswith('w4'):
-            t4, c4 = min(resident)
-            if t4 <= best_t * (1.0 + prefer_resident):
-                best_t, best_comp = t4, c4
-        if prev_comp in times and times[prev_comp] <= best_t * (1.0 + stickiness):
-            best_t, best_comp = times[prev_comp], prev_comp
+        best_comp, best_t = choose_lane(times, prev_comp, stickiness, prefer_resident)
         prev_comp = best_comp
         gain = (orig_t - best_t) * 100 / orig_t if orig_t < float('inf') else 0.0
         perf_list.append((m, best_comp, gain))

@@ -68,6 +68,25 @@ def test_compress_segments_matches_reference_rule():
     assert compress_segments([(1, 'fp16', 1.0)]) == [(1, 'fp16', 1.0)]
 
 
+def test_profiler_lane_choice_rules():
+    """choose_lane: fastest lane; a lane on the resident int4 weight within the margin goes first; the previous M's
+    lane is kept within the stickiness; both margins at zero give the reference's strict minimum
+    (kairos/perf_profiler.py:140-147)."""
+    from kairos_amd.perf_profiler import choose_lane
+    t = {"w8a8": 100.0, "w4a8_qserve": 103.0, "w4a16_gemm": 150.0, "fp16": 170.0}
+    assert choose_lane(t, "", 0.0, 0.0) == ("w8a8", 100.0)
+    assert choose_lane(t, "", 0.01, 0.04) == ("w4a8_qserve", 103.0)          # within 4 %: no converted copy
+    assert choose_lane(t, "", 0.01, 0.02) == ("w8a8", 100.0)                 # beyond the margin: the fastest
+    assert choose_lane({**t, "w4a8_qserve": 104.1}, "", 0.01, 0.04) == ("w8a8", 100.0)
+    assert choose_lane(t, "fp16", 0.01, 0.0) == ("w8a8", 100.0)              # previous lane far behind: dropped
+    assert choose_lane({"w8a8": 100.0, "fp16": 100.5}, "fp16", 0.01, 0.04) == ("fp16", 100.5)   # sticky within 1 %
+    assert choose_lane({"w8a8": 100.0, "fp16": 100.5}, "fp16", 0.0, 0.04) == ("w8a8", 100.0)
+    # stickiness is measured against the choice after the preference, not against the raw minimum
+    assert choose_lane(t, "w8a8", 0.01, 0.04) == ("w8a8", 100.0)
+    assert choose_lane({"w4a16_gemv": 10.0, "w4a16_gemm": 12.0, "w8a8": 30.0}, "", 0.01, 0.04) == ("w4a16_gemv", 10.0)
+    assert choose_lane({"fp16": 5.0}, "w8a8", 0.01, 0.04) == ("fp16", 5.0)   # no resident lane, previous lane absent
+
+
 def test_lut_wrapper():
     from kairos.perf_profiler import LUT
     lut = LUT()
