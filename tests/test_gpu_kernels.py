@@ -316,6 +316,33 @@ def test_gemm_w4a8_bit_exact(ops, M, tile):
     assert_same_bits(host(out_b), out_b_ref)
 
 
+@pytest.mark.parametrize("tile", [128, 130, 192, 256, 512])
+def test_gemm_w4a8_several_ragged_row_tiles(ops, tile):
+    """M = 700 is two 512-row tiles (the second quartet of the second tile lies wholly beyond M), three 256-row tiles
+    and six 128-row tiles, all ragged; N = 640 leaves the 256-column tiles ragged: accumulators and biased fp16
+    outputs against the oracle's W8A8 chain, bit for bit."""
+    M, N, K = 700, 640, 1024
+    p = prep(N, K, seed=tile)
+    x = O.synth_acts(M, K, seed=tile + 1)
+    a8, sx = O.quant_act_i8(x)
+    acc_ref, out_ref = O.gemm_w8a8(a8, p["w8"], p["scales_1"], sx)
+    bias = np.random.default_rng(tile).standard_normal(N).astype(np.float16)
+    out_b_ref = (out_ref.astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    qw, s8, z8 = dev(p["qweight"]), dev(p["scales_to8"]), dev(p["scaled_zeros_to8"])
+    out_b = torch.full((M + 8, N), float("nan"), dtype=torch.float16, device="cuda")     # rows beyond M must stay untouched
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(1)
+    try:
+        acc = ops.w4a8_gemm_acc_i32(dev(a8), qw, s8, z8)
+        ops.w4a8_gemm_forward(dev(a8), qw, s8, z8, dev(p["scales_1"]), dev(sx), out_b[:M], bias=dev(bias))
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert_same_bits(host(acc), acc_ref)
+    assert_same_bits(host(out_b[:M]), out_b_ref)
+    assert torch.isnan(out_b[M:]).all()
+
+
 @pytest.mark.parametrize("tile,splits", [(128, 1), (256, 1), (128, 3), (256, 2), (192, 1), (192, 4), (130, 1), (130, 2), (130, 3), (512, 1), (512, 2), (0, 0)])
 def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
     """Arbitrary tables (every table byte differs from row to row and group to group, values beyond the int8 range are
