@@ -92,11 +92,12 @@ __device__ __forceinline__ void static_for(F&& f) {
 // memory.  Their int32 accumulators meet in LDS at the end (integers: the order does not matter).  Small tiles only:
 // two waves per SIMD leave 256 registers each.
 //
-// MW = 2: two wave quartets on ONE pipeline.  Quartet h multiplies rows h*BM/2 .. of the tile against all BN columns;
-// both read the same LDS stages and all eight waves bring the activation rows in, but only quartet 0 loads, decodes
-// and stores the weights.  With one wave per SIMD every instruction of the stage -- some 200 against 32 MFMAs --
-// queues on that wave's own issue port (one instruction per four cycles), which the MFMAs cannot cover; the second
-// wave of the SIMD issues its MFMAs and fragment reads into those gaps.
+// MW = 2: two wave quartets on ONE pipeline.  Quartet h multiplies rows h*BM/2 .. of the tile against all BN columns and
+// both read the same LDS stages, but the staging is divided: quartet 0 loads, decodes and stores the weights, quartet 1
+// brings in all the activation rows.  With one wave per SIMD every instruction of the stage -- some 200 against 32
+// MFMAs -- queues on that wave's own issue port, which the MFMAs cannot cover, and a 64-lane load holds the port far
+// longer than a vector instruction; with the roles apart the decoding wave never waits behind a load, and the second
+// wave of the SIMD issues its MFMAs, fragment reads and loads into the gaps of the first.
 template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
 __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -107,8 +108,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     constexpr int FM = BMW / 64, FN = BN / 64;
     constexpr int ROWS = BM + BN;
     constexpr int STAGE = ROWS * 64;
-    constexpr int NLA = BM * 4 / (256 * MW);                // direct activation loads per thread and stage
-    constexpr int NLA0 = (NLA + 1) / 2, NLA1 = NLA - NLA0;  // issued behind the barrier / in front of it
+    constexpr int NLA = BM * 4 / 256;                       // direct activation loads per thread and stage, of the quartet that issues them
     constexpr int CPT = BN * 2 / 256;                       // packed 16-byte chunks per thread and stage
     static_assert(BM % 64 == 0 && (BN == 128 || BN == 256) && NLA >= 2, "tile shapes this staging scheme covers");
     using acc_t = i16_t;
@@ -122,7 +122,6 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     const int mh = MW == 2 ? quartet : 0;                    // MW = 2: which half of the tile's rows
     char* const smem = smem_all + kq * (NS * STAGE);         // this quartet's ring (MW = 2: the one ring)
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_all = mh * 4 + wave;                      // among the waves that share the ring
     const int wm = wave >> 1, wn = wave & 1;
     const int M = p.M, N = p.N, K = p.K;
     int tm, tn;
@@ -144,11 +143,12 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-    // ---- activation side: load i of wave w fills the KiB region R = 4*MW*i + w = tile rows 16R .. 16R+15
+    // ---- activation side: load i of wave w fills the KiB region R = 4*i + w = tile rows 16R .. 16R+15 (MW = 2: the
+    // waves of the second quartet, which stage no weights, bring in all the rows of the tile)
     uint32_t voff_a[NLA];
 #pragma unroll
     for (int i = 0; i < NLA; ++i) {
-        const int row = 16 * (4 * MW * i + wave_all) + (lane >> 2);
+        const int row = 16 * (4 * i + wave) + (lane >> 2);
         const int c = (lane & 3) ^ ((row >> 2) & 3);
         int m = m0 + row;
         m = m < M ? m : M - 1;
@@ -174,15 +174,6 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     uint32_t L[4];
 
     auto clamp_stage = [&](int u) { return t0 + (u < T ? u : T - 1); };   // past the end: harmless reloads
-    auto issue_a_half = [&](int u, int slot, int h) {        // h = 0: loads 0 .. NLA0-1, h = 1: the rest
-        char* dst = smem + slot * STAGE + wave_all * 1024;
-        const uint32_t sa = (uint32_t)clamp_stage(u) * 64u;
-#pragma unroll
-        for (int i = 0; i < NLA; ++i) {
-            if ((i < NLA0) != (h == 0)) continue;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * (4096 * MW)), 16, voff_a[i], sa, 0, 0);
-        }
-    };
     auto issue_raw = [&](int u, auto sp, auto gp) {
         const uint32_t sb = (uint32_t)clamp_stage(u) * 128u;
 #pragma unroll
@@ -274,6 +265,17 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     auto pipeline = [&](auto dec_) {
     constexpr bool DEC = decltype(dec_)::value;
     constexpr int CPE = DEC ? CPT : 0, SZ = DEC ? 2 : 0;     // weight-side loads of this wave: packed chunks, scale + zero
+    constexpr int ALD = (MW == 1 || !DEC) ? NLA : 0;         // activation loads of this wave per stage
+    constexpr int NLA0 = (ALD + 1) / 2, NLA1 = ALD - NLA0;   // issued behind the barrier / in front of it
+    auto issue_a_half = [&](int u, int slot, int h) {        // h = 0: loads 0 .. NLA0-1, h = 1: the rest
+        char* dst = smem + slot * STAGE + wave * 1024;
+        const uint32_t sa = (uint32_t)clamp_stage(u) * 64u;
+#pragma unroll
+        for (int i = 0; i < ALD; ++i) {
+            if ((i < NLA0) != (h == 0)) continue;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + i * 4096), 16, voff_a[i], sa, 0, 0);
+        }
+    };
     issue_a_half(0, 0, 0); issue_a_half(0, 0, 1);
     if constexpr (DEC) {
         issue_raw(0, I0{}, I0{});
@@ -292,7 +294,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     issue_a_half(3, 3, 0);
     if constexpr (DEC) issue_raw(3, I1{}, I1{});
     __builtin_amdgcn_sched_barrier(0);
-    wait_vmcnt<NLA + (NLA0 + CPE + SZ) + NLA1 + (NLA0 + CPE)>();
+    wait_vmcnt<ALD + (NLA0 + CPE + SZ) + NLA1 + (NLA0 + CPE)>();
     if constexpr (DEC) {
         static_for<0, 4 + 9 * CPT>([&](auto it) { work_item(I0{}, I0{}, I1{}, it, 0); });       // stage 0 (builds the table)
         static_for<0, 9 * CPT>([&](auto it) { work_item(I1{}, I0{}, I0{}, it, 1); });           // stage 1
@@ -344,14 +346,14 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
             static_for<l0, l1>([&](auto l_) {
                 constexpr int l = decltype(l_)::value;
                 if constexpr (BLK == 0) {                    // second half of the activation rows of stage t+3
-                    char* dst = smem + ((SLOT + 3) & 3) * STAGE + wave_all * 1024;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + (NLA0 + l) * (4096 * MW)), 16, voff_a[NLA0 + l], sa3, 0, 0);
+                    char* dst = smem + ((SLOT + 3) & 3) * STAGE + wave * 1024;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + (NLA0 + l) * 4096), 16, voff_a[NLA0 + l], sa3, 0, 0);
                 } else if constexpr (l < NLA0) {             // first half of the activation rows of stage t+4
-                    char* dst = smem + SLOT * STAGE + wave_all * 1024;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + l * (4096 * MW)), 16, voff_a[l], sa4, 0, 0);
-                } else if constexpr (l < NLA0 + CPT) {       // packed chunks of stage t+4
+                    char* dst = smem + SLOT * STAGE + wave * 1024;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(dst + l * 4096), 16, voff_a[l], sa4, 0, 0);
+                } else if constexpr (l < NLA0 + CPE) {       // packed chunks of stage t+4
                     raw[SP][GP][l - NLA0] = __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b + 16u * (l - NLA0), sb4, 0));
-                } else if constexpr (l == NLA0 + CPT) {      // scale / scaled zero of the group stage t+4 opens
+                } else if constexpr (l == NLA0 + CPE) {      // scale / scaled zero of the group stage t+4 opens
                     sraw[GP] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_s, voff_s, so4, 0);
                 } else {
                     zraw[GP] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_z, voff_s, so4, 0);
