@@ -463,7 +463,7 @@ static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t
 
 // Tile choice by a small cost model fitted to MI355X timings (microseconds).  A 256 x 256 tile over K = 4096 takes
 // about 69.5 us with one workgroup per CU (0.40 of the int8 peak with the decode between the MFMAs); a 256 x 128 tile
-// (selector 192) 0.59 of that (0.54 while every workgroup has a CU to itself), a 128 x 128 tile 0.50 alone on a CU and 0.67 per pair when two share one (its decode
+// (selector 192; eight waves, roles divided as in the 512 x 128 tile) 0.56 of that (0.50 on a single round), a 128 x 128 tile 0.50 alone on a CU and 0.67 per pair when two share one (its decode
 // makes it VALU-bound).  Workgroups run in rounds over the CUs; a split over K divides the tile time and adds the
 // partial-sum traffic and the reduce kernel.  Checked against sweeps of the Llama-3-8B shapes, M = 128 .. 4096:
 // 6144 columns M = 1024 -> 256 x 128 (41.7 us against 48.8 with 128 x 128 and 58.4 with 256 x 256), 28672 columns
@@ -487,11 +487,14 @@ static int w4a8_tile(int M, int N, int K) {
     const Workspace roomy{reinterpret_cast<void*>(16), (size_t)64 << 20};
     const double fixed = 6.0;                                // launch, pipeline fill, epilogue: paid once per launch, split or not
     const double t256 = 63.5 * (double)K / 4096.0;           // + fixed = 69.5 us at K = 4096
-    auto cost = [&](int bm, int bn, double unit_alone, double unit_shared, int shared_cap) {
+    // unit_alone: one round with every CU busy; a round that leaves CUs idle runs faster per workgroup (clock, shared
+    // caches), by `idle_gain` for an empty GPU
+    auto cost = [&](int bm, int bn, double unit_alone, double unit_shared, int shared_cap, double idle_gain = 0.0) {
         const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         const int s = kmi_pick_splits(M, N, K, bm, bn, K >> 7, roomy);
         const long w = tiles * s;
-        const double rounds_t = w <= 256 ? unit_alone : (double)((w + shared_cap - 1) / shared_cap) * unit_shared;
+        const double rounds_t = w <= 256 ? unit_alone - idle_gain * (1.0 - (double)w / 256.0)
+                                         : (double)((w + shared_cap - 1) / shared_cap) * unit_shared;
         double us = fixed + rounds_t * t256 / s;
         if (s > 1) us += (double)(s + 1) * (double)M * (double)N * 4.0 / 4.0e6 + 3.0;
         return us;
@@ -502,7 +505,7 @@ static int w4a8_tile(int M, int N, int K) {
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     const int s128 = kmi_pick_splits(M, N, K, 128, 128, K >> 7, roomy);
     const bool two_quartets = (K % 256 == 0) && tiles128 * s128 <= 256;
-    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.54, 0.59, 256);
+    const double c256 = cost(256, 256, 1.0, 1.0, 256), c192 = cost(256, 128, 0.50, 0.56, 256, 0.25);
     double c128 = cost(128, 128, 0.45, 0.67, 512);
     if (two_quartets) {
         const double w = (double)(tiles128 * s128);
@@ -515,7 +518,7 @@ static int w4a8_tile(int M, int N, int K) {
     if (w4a8_head_cols(M, N) > 0) {
         const int TM = (M + 255) / 256, TN = (N + 255) / 256, head = w4a8_head_cols(M, N);
         const long tail = (long)(TN - head) * TM * 2;
-        c448 = 2.0 * fixed + ((double)(head * TM / 256) + (double)((tail + 255) / 256) * 0.59) * t256;
+        c448 = 2.0 * fixed + ((double)((head * TM + 255) / 256) + (double)((tail + 255) / 256) * 0.55) * t256;
     }
     if (c128 <= c192 && c128 <= c256 && c128 <= c448 && (M < 512 || c128 <= cost(512, 128, 0.90, 0.90, 256))) {
         // At most one workgroup per CU: two wave quartets per workgroup, each on half of the workgroup's K range
@@ -550,10 +553,10 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
     if (tile == 448) {
         const int head = w4a8_head_cols(a.M, a.N) * 256;
         rc = launch_w4a8<KIND, 256, 256>(a, ws, st, 0, head);
-        if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128>(a, ws, st, head, a.N - head);
+        if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
     } else {
         rc = tile == 256 ? launch_w4a8<KIND, 256, 256>(a, ws, st)
-           : tile == 192 ? launch_w4a8<KIND, 256, 128>(a, ws, st)
+           : tile == 192 ? launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st)
            : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st)
            : tile == 512 ? launch_w4a8<KIND, 512, 128, 1, 2>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
     }
