@@ -201,8 +201,8 @@ int kmi_gemm_w8a8_acc_i32(void* acc_i32, const void* a8, const void* w8, int M, 
  * kmi_gemm_w4a8_acc_i32 writes the raw int32 accumulators [M, N] (bit-exact tier).  kmi_gemm_w4a8_pick_tile: host-only,
  * the tile selector the call would use (128 = 128 x 128, 130 = 128 x 128 with two wave quartets per workgroup that
  * each take half of its K range (needs K % 256 == 0), 192 = 256 rows x 128 columns, 512 = 512 rows x 128 columns,
- * 256 = 256 x 256, 448 = 256 x 256
- * tiles in whole rounds over the CUs and the remaining columns as 256 x 128 tiles in a second launch on the same stream);
+ * 256 = 256 x 256, 448 / 640 = 256 x 256 / 512 x 128 tiles in whole rounds over the CUs and the remaining columns as
+ * 256 x 128 tiles in a second launch on the same stream);
  * kmi_gemm_force_tile accepts the same selectors for this lane. */
 int kmi_gemm_w4a8(void* out_f16, const void* a8, const void* qweight, const void* scales_to8, const void* scaled_zeros_to8,
                   const void* wscales_f16, const void* ascales_f16, const void* bias, int M, int N, int K, int G,

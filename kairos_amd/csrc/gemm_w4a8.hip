@@ -479,11 +479,22 @@ static int w4a8_head_cols(int M, int N) {
     return head;
 }
 
+// The same for 512 x 128 tiles (selector 640): column tiles (128 wide) of the whole rounds, when the last round would be
+// at most ~55 % full; the rest runs as 256 x 128 tiles in a second launch.
+static int w4a8_head_cols_512(int M, int N) {
+    const int TM = (M + 511) / 512, TN = (N + 127) / 128;
+    const int tiles = TM * TN, rem = tiles % 256;
+    const int head = (tiles - rem) / TM;
+    if (M < 512 || tiles <= 256 || rem == 0 || head <= 0 || (TN - head) * TM > 140 || (N % 128) != 0) return 0;
+    return head;
+}
+
 static int w4a8_tile(int M, int N, int K) {
     const int forced = kmi_forced_tile();
     if (forced == 128 || forced == 192 || forced == 256 || forced == 512) return forced;
     if (forced == 130) return (K % 256 == 0) ? 130 : 128;    // 128 x 128 tile, two wave quartets per workgroup
     if (forced == 448) return w4a8_head_cols(M, N) > 0 ? 448 : 256;
+    if (forced == 640) return w4a8_head_cols_512(M, N) > 0 ? 640 : 512;
     const Workspace roomy{reinterpret_cast<void*>(16), (size_t)64 << 20};
     const double fixed = 6.0;                                // launch, pipeline fill, epilogue: paid once per launch, split or not
     const double t256 = 63.5 * (double)K / 4096.0;           // + fixed = 69.5 us at K = 4096
@@ -531,6 +542,16 @@ static int w4a8_tile(int M, int N, int K) {
     // against 134.7 us; M=4096: 471 against 488; 6144 columns M=2048: 55.8 against 61.9; four waves of 256 x 64 each on
     // the same tile: 127.5 / 475 / 58.3).  Not below 512 rows, where half of the tile would be padding.
     const double c512 = M >= 512 ? cost(512, 128, 0.90, 0.90, 256) : 1e30;
+    // whole rounds of 512 x 128 tiles + the columns of a thin last round as 256 x 128 tiles (selector 640): 2048 x 28672 is
+    // 3.5 rounds -> 3 rounds + 256 half-size workgroups
+    double c640 = 1e30;
+    if (w4a8_head_cols_512(M, N) > 0) {
+        const int TM = (M + 511) / 512, TN = (N + 127) / 128, head = w4a8_head_cols_512(M, N);
+        const long tail = (long)(TN - head) * ((M + 255) / 256);
+        const double tail_unit = tail <= 256 ? 0.50 - 0.25 * (1.0 - (double)tail / 256.0) : (double)((tail + 255) / 256) * 0.56;
+        c640 = 2.0 * fixed + ((double)((head * TM + 255) / 256) * 0.90 + tail_unit) * t256;
+    }
+    if (c640 < c512 && c640 < c448 && c640 < c192 && c640 < c256) return 640;
     if (c512 < c448 && c512 < c192 && c512 < c256) return 512;
     if (c448 <= c192 && c448 <= c256) return 448;
     return c192 <= c256 ? 192 : 256;
@@ -550,7 +571,11 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
     if (a.M == 0) return KMI_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int tile = w4a8_tile(a.M, a.N, a.K);
-    if (tile == 448) {
+    if (tile == 640) {
+        const int head = w4a8_head_cols_512(a.M, a.N) * 128;
+        rc = launch_w4a8<KIND, 512, 128, 1, 2>(a, ws, st, 0, head);
+        if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
+    } else if (tile == 448) {
         const int head = w4a8_head_cols(a.M, a.N) * 256;
         rc = launch_w4a8<KIND, 256, 256>(a, ws, st, 0, head);
         if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st, head, a.N - head);

@@ -373,8 +373,9 @@ def gemm_tile_for(M, N, K=4096):
 
 
 def gemm_w4a8_tile_for(M, N, K=4096):
-    """Tile selector of the W4A8 GEMM for an M x N x K product: 128 (128 x 128), 192 (256 x 128), 256 (256 x 256) or 448
-    (256 x 256 in whole rounds, the remaining columns as 256 x 128 tiles in a second launch)."""
+    """Tile selector of the W4A8 GEMM for an M x N x K product: 128 (128 x 128), 130 (the same on two wave quartets),
+    192 (256 x 128), 256 (256 x 256), 512 (512 x 128), 448 / 640 (256 x 256 / 512 x 128 in whole rounds, the remaining
+    columns as 256 x 128 tiles in a second launch)."""
     return _lib.load().kmi_gemm_w4a8_pick_tile(int(M), int(N), int(K))
 
 

@@ -343,6 +343,39 @@ def test_gemm_w4a8_several_ragged_row_tiles(ops, tile):
     assert torch.isnan(out_b[M:]).all()
 
 
+@pytest.mark.parametrize("sel,M,N", [(640, 520, 19200), (448, 300, 38400)])
+def test_gemm_w4a8_whole_rounds_plus_a_tail_launch(ops, sel, M, N):
+    """More tiles than compute units with a thin last round: the columns of the whole rounds run as one launch of the
+    large tile (512 x 128: 2 x 150 = 300 tiles -> 128 column tiles; 256 x 256: 2 x 150 -> 128), the remaining columns as
+    256 x 128 tiles in a second launch.  The seam must not show: outputs equal the 128 x 128 kernel's bit for bit, and
+    the oracle's on sampled rows."""
+    K = 256
+    p = prep(N, K, seed=sel)
+    x = O.synth_acts(M, K, seed=sel + 1)
+    a8_np, sx_np = O.quant_act_i8(x)
+    bias_np = np.random.default_rng(sel).standard_normal(N).astype(np.float16)
+    a8, sx, bias = dev(a8_np), dev(sx_np), dev(bias_np)
+    qw, s8, z8, s1 = dev(p["qweight"]), dev(p["scales_to8"]), dev(p["scaled_zeros_to8"]), dev(p["scales_1"])
+    got = {}
+    for tile in (sel, 128):
+        ops.force_gemm_tile(tile)
+        try:
+            if tile == sel:
+                assert ops.gemm_w4a8_tile_for(M, N, K) == sel          # the split applies to this shape
+            acc = ops.w4a8_gemm_acc_i32(a8, qw, s8, z8)
+            out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            ops.w4a8_gemm_forward(a8, qw, s8, z8, s1, sx, out, bias=bias)
+            got[tile] = (acc, out)
+        finally:
+            ops.force_gemm_tile(0)
+    assert torch.equal(got[sel][0], got[128][0]) and torch.equal(got[sel][1], got[128][1])
+    rows = np.array([0, 1, 255, 256, M - 1])
+    acc_ref, out_ref = O.gemm_w8a8(a8_np[rows], p["w8"], p["scales_1"], sx_np[rows])
+    assert_same_bits(host(got[sel][0])[rows], acc_ref)
+    ref_b = (out_ref.astype(np.float32) + bias_np.astype(np.float32)).astype(np.float16)
+    assert_same_bits(host(got[sel][1])[rows], ref_b)
+
+
 @pytest.mark.parametrize("K", [128, 256, 384])
 @pytest.mark.parametrize("tile", [128, 130, 192, 256, 512])
 def test_gemm_w4a8_k_shorter_than_the_pipeline(ops, tile, K):
