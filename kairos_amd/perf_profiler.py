@@ -191,7 +191,7 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
                 cache.invalidate()
                 copies[i % len(copies)]._forward(x, m, cid)
             rec = []
-            if head_start_ms > 0:
+            if head_start_ms > 0 and hasattr(torch.cuda, "_sleep"):
                 torch.cuda._sleep(int(head_start_ms * 2.4e6))          # ~2.4 counts per nanosecond on this part
             with timer(comp, n=n, recordList=rec, print_flag=print_flag):
                 for i in range(n):
