@@ -167,7 +167,8 @@ def test_perf(proj_name, K, N, bias, input_len=None, comp_type_list=None, n=200,
     del lin
     copies = [dlinear]
     weight_bytes = dlinear.qweight.numel() * dlinear.qweight.element_size()
-    for _ in range(min(16, -(-rotate_bytes // weight_bytes)) - 1 if rotate_bytes else 0):
+    rotate = rotate_bytes > 0 and not getattr(linear_cls, "resident_copies", False)   # a layer with resident converted copies is not cloned
+    for _ in range(min(16, -(-rotate_bytes // weight_bytes)) - 1 if rotate else 0):
         twin = linear_cls(K, N, bias, 'cuda', dlinear.group_size)
         for key, value in dlinear.named_buffers():
             setattr(twin, key, value.clone() if key == 'qweight' else value)
