@@ -65,6 +65,14 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_gemm_pick_tile(768, 8192, 28672) == 256 and lib.kmi_gemm_pick_tile(1024, 4096, 14336) == 128   # split over K counts on long rows only
     assert lib.kmi_gemm_pick_tile(2048, 4096, 14336) == 192 and lib.kmi_gemm_pick_tile(1024, 8192, 28672) == 256   # 256 x 128 tiles, two per CU
     assert lib.kmi_gemm_pick_tile(192, 10240, 8192) == 64 and lib.kmi_gemm_pick_tile(192, 28672, 4096) == 128      # row padding
+    # tile choice of the W4A8 GEMM is host logic as well (a cost model fitted to MI355X timings): two wave quartets on
+    # 128 x 128 tiles while at most one workgroup per CU, 256 x 128 in between, 512 x 128 from full rounds on, whole rounds
+    # plus a tail launch where the last round would be thin; two quartets over K need K % 256 == 0
+    picks = {(128, 28672, 4096): 130, (256, 28672, 4096): 192, (512, 28672, 4096): 512, (2048, 28672, 4096): 640,
+             (4096, 28672, 4096): 512, (768, 4096, 14336): 130, (2048, 4096, 14336): 192, (4096, 4096, 14336): 512,
+             (512, 6144, 4096): 130, (1024, 6144, 4096): 192, (128, 4096, 4224): 192}
+    for (M, N, K), want in picks.items():
+        assert lib.kmi_gemm_w4a8_pick_tile(M, N, K) == want, (M, N, K)
     # offline weight preparation: same shape rules as the converters; table height is host arithmetic
     assert lib.kmi_prepare_weight(None, 8, 128, 128, 16, 16, 16, 16, 16, 16, None) == -1
     assert lib.kmi_prepare_weight(16, 6, 128, 128, 16, 16, 16, 16, 16, 16, None) == -2
