@@ -152,12 +152,34 @@ int kmi_gemv_w4a16(void* out_f16, const void* x_f16, const void* qweight, const 
                    const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
                    void* workspace, size_t workspace_bytes, void* stream);
 
-/* Tuning variant: nt = 16-column tiles per wave (1..8), nw = waves per workgroup (4,8,16), ks = workgroups that share
- * the K range of one column strip (1 = no split; more needs a workspace of KMI_GEMV_WS_HEADER + ks*M*N*4 bytes);
- * nt<=0 or nw<=0 selects the built-in heuristic for all three.  No reference counterpart. */
+/* Tuning variant of the register form (a wave keeps the K groups of a trip in registers): nt = 16-column tiles per wave
+ * (1..8), nw = waves per workgroup (4,8,16), ks = workgroups that share the K range of one column strip (1 = no split;
+ * more needs a workspace of KMI_GEMV_WS_HEADER + ks*M*N*4 bytes); nt<=0 or nw<=0 selects the built-in choice of form
+ * and split (what kmi_gemv_w4a16 runs).  No reference counterpart. */
 int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
                        const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
                        int nt, int nw, int ks, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Tuning variant of the ring form: every operand of a K group travels global -> LDS by direct-to-LDS buffer loads into
+ * a per-wave ring of `depth` slots, so loads for later groups stay in flight while a group is multiplied.  nt as above,
+ * nw = 1, 2, 4 or 8, ks as above, depth = slots per wave (<= 0: as deep as the wave's share of K, the wait counter and
+ * LDS allow; larger values are reduced to that).  Same arithmetic and summation order as the register form with the
+ * same (nt, nw, ks).  Needs 4-byte aligned tables and operands below 4 GiB.  No reference counterpart. */
+int kmi_gemv_w4a16_ring_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                            const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                            int nt, int nw, int ks, int depth, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Host only: what kmi_gemv_w4a16 does for this shape with a workspace of that many bytes (0 = none).  *form: 0 register
+ * form, 1 ring form; *nt, *nw, *ks as above; *depth: ring slots asked for (0 for the register form).  Any output pointer
+ * may be NULL. */
+int kmi_gemv_w4a16_plan(int M, int N, int K, size_t workspace_bytes, int* form, int* nt, int* nw, int* ks, int* depth);
+
+/* Writes zeros over the arrival counters of a small-M workspace (its first KMI_GEMV_WS_HEADER bytes) with a small
+ * kernel on `stream`.  Needed once before a buffer's first use unless it was allocated zeroed, and after any call on it
+ * that did not run to completion (a launch error, an aborted stream): counters left non-zero would make later split
+ * calls on that buffer add their partial sums at the wrong arrival.  A kernel, not a memset, so the call can be
+ * captured into a graph.  No reference counterpart. */
+int kmi_gemv_ws_reset(void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- MFMA GEMMs, any M -------------------------------------------------------------------------
  *

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libkairos_mi.so")
 _P = ctypes.c_void_p
 _I = ctypes.c_int
 _Z = ctypes.c_size_t
+_IP = ctypes.POINTER(ctypes.c_int)
 
 # name -> argument types (every function returns int unless listed in _RESTYPE)
 SIGNATURES = {
@@ -31,6 +32,9 @@ SIGNATURES = {
     "kmi_trans_layout_w4a8": [_P, _P, _I, _I, _P],
     "kmi_gemv_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemv_w4a16_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemv_w4a16_ring_cfg": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemv_w4a16_plan": [_I, _I, _I, _Z, _IP, _IP, _IP, _IP, _IP],
+    "kmi_gemv_ws_reset": [_P, _Z, _P],
     # GEMMs end with (workspace pointer, workspace bytes, stream)
     "kmi_gemm_w4a16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w4a16_noalloc": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

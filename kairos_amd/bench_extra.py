@@ -446,16 +446,18 @@ class Decoder:
         self.pos.fill_(prompt_len)
 
     def capture(self):
-        """One warm-up step on a side stream, then the step recorded on that stream (its split-K scratch and the
-        temp cache exist by then).  The caller re-starts the sequence afterwards."""
+        """One warm-up step on a side stream, then the step recorded on that stream (the temp cache exists by then).
+        The captured kernels use a scratch of their own, so a replay never shares split-K partial sums with eager
+        work.  The caller re-starts the sequence afterwards."""
+        self.scratch = ops.Scratch(self.dev)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
+        with torch.cuda.stream(side), self.scratch:
             self.step()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, stream=side):
+        with self.scratch, torch.cuda.graph(self.graph, stream=side):
             self.step()
         return self.graph
 

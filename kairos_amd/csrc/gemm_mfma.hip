@@ -796,6 +796,7 @@ extern "C" void kmi_gemm_force_splits(int splits) { g_force_splits = splits; }
 // two is 1.3-2x slower than running them as they are.
 int kmi_pick_splits(int M, int N, int K, int BM, int BN, int ktiles, const Workspace& ws) {
     const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    if (tiles <= 0) return 1;                                 // empty product (M or N not positive): nothing to split
     int s = 1;
     if (g_force_splits > 0) {
         s = g_force_splits;
@@ -930,6 +931,7 @@ static int launch_w4a16_wp(const GemmArgs& a_in, const Workspace& ws, hipStream_
 //   * where 128-row tiles pad M further than 64-row tiles and would not fill the GPU while the 64-row tiles do,
 //     the latter win (192 x 10240 x 8192: 28.8 against 31.9 us; not at 192 x 28672 x 4096: 52.5 against 43.7 us).
 static int pick_tile(int M, int N, long row_bytes) {
+    if (M <= 0 || N <= 0) return 64;                          // empty product: the entry points return before any launch
     auto wgs = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (row_bytes <= 0) {
         if (M > 128 && wgs(256, 256) >= 180) return 256;

@@ -21,8 +21,6 @@ struct GemmArgs {
     int n_begin, n_cols;      // output columns this launch covers (a multiple of the tile width unless it ends at N)
 };
 
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
 

@@ -490,6 +490,7 @@ static int w4a8_head_cols_512(int M, int N) {
 }
 
 static int w4a8_tile(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 128;              // empty product: the entry points return before any launch
     const int forced = kmi_forced_tile();
     if (forced == 128 || forced == 192 || forced == 256 || forced == 512) return forced;
     if (forced == 130) return (K % 256 == 0) ? 130 : 128;    // 128 x 128 tile, two wave quartets per workgroup

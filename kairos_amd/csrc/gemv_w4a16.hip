@@ -30,6 +30,80 @@
 // matching A fragment is x[m = r16][same eight k], one 16-byte load.  Four MFMAs (a = 0..3) per tile
 // consume the group.
 #include "kmi_common.h"
+#include <mutex>
+#include <set>
+
+// Tail shared by the kernels of this file: the waves' partial tiles meet in LDS (`red`, nw * MT*NT*4 * 64 floats)
+// and are added in wave order; with a split over K (gridDim.y > 1) the workgroup's sums go to `partial`, the
+// strip's arrival counter is bumped and whichever workgroup arrives last adds the slices in split order.
+template <int MT, int NT>
+__device__ __forceinline__ void gemv_finish(const f4_t (&acc)[MT][NT], float* red, int NW, int wave, int lane, int strip, int n0,
+                                            half_t* __restrict__ out, const half_t* __restrict__ bias, int M, int N,
+                                            float* __restrict__ partial, uint32_t* __restrict__ counters) {
+    const int KS = gridDim.y, ks = blockIdx.y;
+    constexpr int R = MT * NT * 4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[(wave * R + (mt * NT + nt) * 4 + i) * 64 + lane] = acc[mt][nt][i];
+    __syncthreads();
+
+    if (KS == 1) {
+        for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
+            const int l = idx & 63, reg = idx >> 6;
+            const int i = reg & 3, t = reg >> 2;
+            const int nt = t % NT, mt = t / NT;
+            const int m = mt * 16 + 4 * (l >> 4) + i;
+            const int n = n0 + nt * 16 + (l & 15);
+            if (m < M && n < N) {
+                half_t h = (half_t)v;
+                if (bias) h = (half_t)((float)h + (float)bias[n]);
+                out[(long)m * N + n] = h;
+            }
+        }
+        return;
+    }
+    // ---- K split over workgroups: publish this workgroup's partial sums, count the arrival, last one finishes
+    for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
+        const int l = idx & 63, reg = idx >> 6;
+        const int i = reg & 3, t = reg >> 2;
+        const int nt = t % NT, mt = t / NT;
+        const int m = mt * 16 + 4 * (l >> 4) + i;
+        const int n = n0 + nt * 16 + (l & 15);
+        if (m < M && n < N)
+            __hip_atomic_store(partial + ((long)ks * M + m) * N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this thread's partial sums have been performed
+    __shared__ uint32_t arrived;
+    __syncthreads();                                         // ... and everybody else's in the workgroup
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counters + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrived != (uint32_t)(KS - 1)) return;               // workgroup-uniform
+    for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
+        const int l = idx & 63, reg = idx >> 6;
+        const int i = reg & 3, t = reg >> 2;
+        const int nt = t % NT, mt = t / NT;
+        const int m = mt * 16 + 4 * (l >> 4) + i;
+        const int n = n0 + nt * 16 + (l & 15);
+        if (m < M && n < N) {
+            float v = 0.f;
+            for (int q = 0; q < KS; ++q)                     // split order: the same sum whoever arrives last
+                v += __hip_atomic_load(partial + ((long)q * M + m) * N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            half_t h = (half_t)v;
+            if (bias) h = (half_t)((float)h + (float)bias[n]);
+            out[(long)m * N + n] = h;
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+}
 
 template <int MT, int NT, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict__ out, const half_t* __restrict__ x,
@@ -157,68 +231,185 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
         }
     }
 
-    constexpr int R = MT * NT * 4;
+    gemv_finish<MT, NT>(acc, red, NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
+}
+
+// =====================================================================================================================
+// Ring form of the same product.  Registers cannot hold more than one or two K groups per wave in flight, so the
+// kernel above alternates between waiting for HBM and computing.  Here every operand of a K group -- NT KiB of packed
+// weights, the activation rows, the group's scale-table entries -- travels global -> LDS by buffer loads that write
+// LDS directly (no destination registers), into a ring of D slots that is private to the wave: the wave keeps D groups
+// in flight, waits with `s_waitcnt vmcnt` for the oldest (loads retire in issue order), copies it to registers,
+// re-issues the slot for the group D trips ahead and only then computes.  No barrier until the final reduction.
+//   slot = [NT x 1 KiB weights: lane l's 16-byte chunk at l*16][XI x 1 KiB activations][256 B scales][256 B scaled zeros]
+//   activations: 16-byte unit `ch` (0..15) of row r of the group's [rows][128] block sits at unit r*16 + (ch ^ (r & 15)),
+//   so the 16 lanes that read one plane of 16 different rows hit 16 different bank quads; XI loads cover 4*XI rows
+//   (rows >= M repeat row M-1: their products land in output rows that are never stored).
+template <int L, int KMAX>
+__device__ __forceinline__ void gemv_wait_slots(int k) {         // until at most k slots' loads (L each) are outstanding
+    if constexpr (KMAX > 0) {
+        if (k >= KMAX) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KMAX * L) : "memory");
+            return;
+        }
+        gemv_wait_slots<L, KMAX - 1>(k);
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+}
+
+template <int XI, int NT>
+static constexpr int gemv_ring_max_depth() {                        // vmcnt counts up to 63
+    constexpr int L = NT + XI + 2;
+    return (63 / L + 1) < 8 ? (63 / L + 1) : 8;
+}
+
+template <int XI, int NT>
+__global__ __launch_bounds__(512) void gemv_ring_kernel(half_t* __restrict__ out, const half_t* __restrict__ x,
+                                                        const u4_t* __restrict__ qw, const half_t* __restrict__ scales,
+                                                        const half_t* __restrict__ szeros, const half_t* __restrict__ bias,
+                                                        int M, int N, int K, int D, float* __restrict__ partial,
+                                                        uint32_t* __restrict__ counters) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass cannot instantiate code that uses the buffer resource type
+    constexpr int MT = (XI + 3) / 4;
+    constexpr int L = NT + XI + 2;                                 // direct loads per slot
+    constexpr int X_OFF = NT * 1024, S_OFF = X_OFF + XI * 1024, SLOT = S_OFF + 512;
+    constexpr int KMAX = gemv_ring_max_depth<XI, NT>() - 1;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: feeds M0
+    const int NW = blockDim.x >> 6;
+    const int r16 = lane & 15, j = lane >> 4;
+    const int nblk = gridDim.x, xcd = blockIdx.x & 7;               // contiguous run of strips per XCD, as above
+    const int strip = xcd * (nblk >> 3) + min(xcd, nblk & 7) + (blockIdx.x >> 3);
+    const int n0 = strip * (16 * NT);
+    const int KS = gridDim.y, ks = blockIdx.y;
+    const int all_groups = K >> 7;
+    const int g0 = (int)((long)ks * all_groups / KS), g1 = (int)((long)(ks + 1) * all_groups / KS);
+    const int kq = K >> 3;
+    const int mine = g0 + wave < g1 ? (g1 - g0 - wave + NW - 1) / NW : 0;   // groups g0 + wave + i*NW, i < mine
+
+    // ---- global sources: a resource per tensor, a per-lane byte offset that never changes, a scalar offset per group
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<u4_t*>(qw), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(scales), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(szeros), 0, -1, 0x00020000);
+    uint32_t voff_w[NT], voff_x[XI];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int n = n0 + nt * 16 + r16;
+        n = n < N ? n : N - 1;                                     // partial last strip: clamp loads, stores are masked
+        voff_w[nt] = (uint32_t)(((long)(n >> 2) * kq + (n & 3) * 2 + (j & 1) + (j >> 1) * 8) * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const int p = i * 64 + lane, row = p >> 4, ch = (p & 15) ^ (row & 15);
+        const int m = row < M ? row : M - 1;
+        voff_x[i] = (uint32_t)(((long)m * K + ch * 8) * 2);
+    }
+    uint32_t voff_s;
+    {
+        int n = n0 + 2 * (lane < 8 * NT ? lane : 8 * NT - 1);
+        n = n < N ? n : N - 2;
+        voff_s = (uint32_t)(n * 2);
+    }
+    char* ring = smem + wave * (D * SLOT);
+    auto issue = [&](int slot, int i) {                             // the wave's i-th group into ring slot `slot`
+        const uint32_t c = (uint32_t)(g0 + wave + i * NW);
+        char* dst = ring + slot * SLOT;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_void_ptr)(dst + nt * 1024), 16, voff_w[nt], c * 256u, 0, 0);
+#pragma unroll
+        for (int t = 0; t < XI; ++t)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_void_ptr)(dst + X_OFF + t * 1024), 16, voff_x[t], c * 256u, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_s, (lds_void_ptr)(dst + S_OFF), 4, voff_s, c * (uint32_t)(N * 2), 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_z, (lds_void_ptr)(dst + S_OFF + 256), 4, voff_s, c * (uint32_t)(N * 2), 0, 0);
+    };
+
+    // ---- LDS read addresses of this lane inside a slot
+    int xoff[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int row = mt * 16 + r16;
+        row = row < 4 * XI ? row : 4 * XI - 1;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) xoff[mt][a] = X_OFF + (row * 16 + ((4 * j + a) ^ (row & 15))) * 16;
+    }
+
+    f4_t acc[MT][NT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) red[(wave * R + (mt * NT + nt) * 4 + i) * 64 + lane] = acc[mt][nt][i];
-    __syncthreads();
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const h8_t ones = {(half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1};
+    const h8_t sixteenth = ones * (half_t)0.0625f;
 
-    if (KS == 1) {
-        for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
-            float v = 0.f;
+    const int pre = mine < D ? mine : D;
+    for (int i = 0; i < pre; ++i) issue(i, i);
+    int slot = 0;
+    for (int i = 0; i < mine; ++i) {
+        const int behind = mine - 1 - i;                            // slots issued after this one and still wanted
+        gemv_wait_slots<L, KMAX>(behind < D - 1 ? behind : D - 1);
+        const char* src = ring + slot * SLOT;
+        u4_t u[NT];
+        half_t sc_h[NT], zc_h[NT];
+        h8_t xa[MT][4];
 #pragma unroll
-            for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
-            const int l = idx & 63, reg = idx >> 6;
-            const int i = reg & 3, t = reg >> 2;
-            const int nt = t % NT, mt = t / NT;
-            const int m = mt * 16 + 4 * (l >> 4) + i;
-            const int n = n0 + nt * 16 + (l & 15);
-            if (m < M && n < N) {
-                half_t h = (half_t)v;
-                if (bias) h = (half_t)((float)h + (float)bias[n]);
-                out[(long)m * N + n] = h;
+        for (int nt = 0; nt < NT; ++nt) {
+            u[nt] = *reinterpret_cast<const u4_t*>(src + nt * 1024 + lane * 16);
+            sc_h[nt] = *reinterpret_cast<const half_t*>(src + S_OFF + (nt * 16 + r16) * 2);
+            zc_h[nt] = *reinterpret_cast<const half_t*>(src + S_OFF + 256 + (nt * 16 + r16) * 2);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) xa[mt][a] = *reinterpret_cast<const h8_t*>(src + xoff[mt][a]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");         // the slot is in registers: hand it back
+        if (i + D < mine) issue(slot, i + D);
+        slot = slot + 1 == D ? 0 : slot + 1;
+
+        f4_t xsum[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            xsum[mt] = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][a], ones, xsum[mt], 0, 0, 0);
+            xa[mt][1] *= sixteenth;                                 // planes 1 and 3 carry 16q
+            xa[mt][3] *= sixteenth;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            u4_t lo, hi, lo8, hi8;                                  // nibble planes 0, 1, 2, 3 as fp16 subnormals
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t v = u[nt][w], v8 = v >> 8;
+                lo[w] = v & 0x000F000Fu;
+                hi[w] = v & 0x00F000F0u;
+                lo8[w] = v8 & 0x000F000Fu;
+                hi8[w] = v8 & 0x00F000F0u;
+            }
+            const float sc = (float)sc_h[nt] * 16777216.0f;         // undo the 2^-24 of the subnormal encoding
+            const float zc = (float)zc_h[nt];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                f4_t pg = {0.f, 0.f, 0.f, 0.f};
+                pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][0], __builtin_bit_cast(h8_t, lo), pg, 0, 0, 0);
+                pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][1], __builtin_bit_cast(h8_t, hi), pg, 0, 0, 0);
+                pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][2], __builtin_bit_cast(h8_t, lo8), pg, 0, 0, 0);
+                pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][3], __builtin_bit_cast(h8_t, hi8), pg, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[mt][nt][e] = __builtin_fmaf(pg[e], sc, __builtin_fmaf(xsum[mt][e], zc, acc[mt][nt][e]));
             }
         }
-        return;
     }
-    // ---- K split over workgroups: publish this workgroup's partial sums, count the arrival, last one finishes
-    for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
-        float v = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
-        const int l = idx & 63, reg = idx >> 6;
-        const int i = reg & 3, t = reg >> 2;
-        const int nt = t % NT, mt = t / NT;
-        const int m = mt * 16 + 4 * (l >> 4) + i;
-        const int n = n0 + nt * 16 + (l & 15);
-        if (m < M && n < N)
-            __hip_atomic_store(partial + ((long)ks * M + m) * N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this thread's partial sums have been performed
-    __shared__ uint32_t arrived;
-    __syncthreads();                                         // ... and everybody else's in the workgroup
-    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counters + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // every wave has emptied its ring (and no direct load is outstanding) before the rings become the reduction buffer
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    if (arrived != (uint32_t)(KS - 1)) return;               // workgroup-uniform
-    for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
-        const int l = idx & 63, reg = idx >> 6;
-        const int i = reg & 3, t = reg >> 2;
-        const int nt = t % NT, mt = t / NT;
-        const int m = mt * 16 + 4 * (l >> 4) + i;
-        const int n = n0 + nt * 16 + (l & 15);
-        if (m < M && n < N) {
-            float v = 0.f;
-            for (int q = 0; q < KS; ++q)                     // split order: the same sum whoever arrives last
-                v += __hip_atomic_load(partial + ((long)q * M + m) * N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            half_t h = (half_t)v;
-            if (bias) h = (half_t)((float)h + (float)bias[n]);
-            out[(long)m * N + n] = h;
-        }
-    }
-    if (threadIdx.x == 0) __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+    gemv_finish<MT, NT>(acc, reinterpret_cast<float*>(smem), NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
+#endif
 }
 
 typedef void (*gemv_fn)(half_t*, const half_t*, const u4_t*, const half_t*, const half_t*, const half_t*, int, int, int, float*, uint32_t*);
@@ -324,9 +515,87 @@ static void gemv_default_cfg(int M, int mt, int N, int K, int* nt_out, int* nw_o
     }
 }
 
-extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
-                                  const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
-                                  int nt, int nw, int ks, void* workspace, size_t workspace_bytes, void* stream) {
+// ---- ring form: dispatch over (activation loads per group, column tiles per wave) -------------------------------------
+typedef void (*gemv_ring_fn)(half_t*, const half_t*, const u4_t*, const half_t*, const half_t*, const half_t*, int, int, int, int,
+                             float*, uint32_t*);
+struct GemvRingKernel { gemv_ring_fn fn; int slot_bytes, max_depth; };
+
+template <int XI, int NT>
+static GemvRingKernel gemv_ring_pick() {
+    if constexpr (((XI + 3) / 4) * NT <= 8) return {gemv_ring_kernel<XI, NT>, NT * 1024 + XI * 1024 + 512, gemv_ring_max_depth<XI, NT>()};
+    else return {nullptr, 0, 0};
+}
+
+template <int XI>
+static GemvRingKernel gemv_ring_pick_nt(int nt) {
+    switch (nt) {
+        case 1: return gemv_ring_pick<XI, 1>();
+        case 2: return gemv_ring_pick<XI, 2>();
+        case 3: return gemv_ring_pick<XI, 3>();
+        case 4: return gemv_ring_pick<XI, 4>();
+        case 5: return gemv_ring_pick<XI, 5>();
+        case 6: return gemv_ring_pick<XI, 6>();
+        case 7: return gemv_ring_pick<XI, 7>();
+        case 8: return gemv_ring_pick<XI, 8>();
+    }
+    return {nullptr, 0, 0};
+}
+
+static int gemv_ring_xi(int M) { return M <= 4 ? 1 : M <= 8 ? 2 : M <= 16 ? 4 : M <= 32 ? 8 : M <= 48 ? 12 : 16; }
+
+static GemvRingKernel gemv_ring_lookup(int M, int nt) {
+    switch (gemv_ring_xi(M)) {
+        case 1: return gemv_ring_pick_nt<1>(nt);
+        case 2: return gemv_ring_pick_nt<2>(nt);
+        case 4: return gemv_ring_pick_nt<4>(nt);
+        case 8: return gemv_ring_pick_nt<8>(nt);
+        case 12: return gemv_ring_pick_nt<12>(nt);
+        case 16: return gemv_ring_pick_nt<16>(nt);
+    }
+    return {nullptr, 0, 0};
+}
+
+// When the ring form runs, and with which split (graph-replay timings on MI355X, us, register form -> ring form;
+// weights rotated through 700 MB):
+//   M > 16 (two or more row tiles): always.  4096 x 4096 M=32 9.8 -> 8.1, 6144 x 4096 11.0 -> 9.0, 28672 x 4096 24.6 ->
+//   23.2, 4096 x 14336 18.5 -> 16.6, 10240 x 8192 20.5 -> 17.2, 57344 x 8192 80 -> 72, 8192 x 28672 41.7 -> 38.4,
+//   3584 x 18944 31.1 -> 19.4.  Column tiles per wave: one per 256 strips (so that about one workgroup lands on each
+//   CU), as many as the accumulators allow beyond.
+//   M <= 16 on narrow weights (at most 320 column strips) from M = 8, or from M = 1 where K is long (>= 96 groups):
+//   4096 x 4096 M=8 5.8 -> 5.5, M=16 6.7 -> 6.2; 4608 x 3584 M=16 7.2 -> 6.6; 4096 x 14336 M=1 9.9 -> 9.5, M=16 12.8 ->
+//   12.2; 3584 x 18944 M=16 19.4 -> 14.3.  Wide weights (28672, 37888, 57344 columns) stay with the register form there
+//   (12.8 against 14.6 us at 28672 x 4096): their trips are long enough to cover the wait, and the ring's extra hop
+//   through LDS costs more than it hides.
+//   Long K (>= 96 groups) at M >= 8: two workgroups share a strip's K range and the waves take twice the column tiles,
+//   which halves the activation bytes every CU pulls through its L1.
+static bool gemv_ring_default(int M, int N, int K, bool can_split, int* nt, int* nw, int* ks, int* depth) {
+    const int strips = N / 16, groups = K / 128, mt = (M + 15) / 16, cap = 8 / mt;
+    int per_round = (strips + 255) / 256;
+    if (per_round > cap) per_round = cap;
+    *nw = 8;
+    *depth = 2;
+    *ks = 1;
+    *nt = per_round;
+    const bool long_k = can_split && groups >= 96 && strips <= 512;    // without scratch for a split: the unsplit ring
+    if (M > 16) {
+        if (long_k) {
+            *nt = 2 * per_round < cap ? 2 * per_round : cap;
+            *ks = 2;
+        }
+        return true;
+    }
+    if (strips > 320 || !(M >= 8 || groups >= 96)) return false;
+    if (M >= 8 && long_k) {
+        *nt = 2;
+        *ks = 2;
+    }
+    return true;
+}
+
+#define KMI_GEMV_RING_LDS (160 * 1024 - 256)   // dynamic LDS a workgroup may ask for: the CU's 160 KiB less the static part (arrival flag)
+
+static int gemv_check_args(const void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                           const void* scaled_zeros, int M, int N, int K, int G, const void* workspace) {
     if (!out_f16 || !x_f16 || !qweight || !scales || !scaled_zeros)
         return kmi_set_error(KMI_E_NULL, "kmi_gemv_w4a16: NULL pointer argument");
     if (!kmi_aligned16(x_f16) || !kmi_aligned16(qweight) || (workspace && !kmi_aligned16(workspace)))
@@ -336,9 +605,120 @@ extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* 
         return kmi_set_error(KMI_E_M_RANGE, "kmi_gemv_w4a16: M=%d outside 1..%d", M, KMI_GEMV_MAX_M);
     if (N <= 0 || K <= 0 || (N & 15) || (K & 127))
         return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: need N%%16==0 and K%%128==0, got N=%d K=%d", N, K);
+    return KMI_OK;
+}
+
+// The ring form addresses its operands with 32-bit buffer offsets and loads table entries as dwords.
+static bool gemv_ring_eligible(const void* scales, const void* scaled_zeros, int M, int N, int K) {
+    return !(reinterpret_cast<uintptr_t>(scales) & 3u) && !(reinterpret_cast<uintptr_t>(scaled_zeros) & 3u) &&
+           (long)N * K / 2 < (1L << 32) && (long)M * K * 2 < (1L << 32) && (long)(K / 128) * N * 2 < (1L << 32);
+}
+
+static int gemv_ring_launch(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                            const void* scaled_zeros, const void* bias, int M, int N, int K,
+                            int nt, int nw, int ks, int depth, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!gemv_ring_eligible(scales, scaled_zeros, M, N, K))
+        return kmi_set_error(KMI_E_ALIGN, "kmi_gemv_w4a16: the ring form needs 4-byte aligned tables and operands below 4 GiB");
+    const GemvRingKernel kn = gemv_ring_lookup(M, nt);
+    if (!kn.fn || (nw != 1 && nw != 2 && nw != 4 && nw != 8))
+        return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: no ring kernel for M=%d nt=%d nw=%d", M, nt, nw);
+    const int strips = N / 16, wg_x = (strips + nt - 1) / nt, groups = K / 128;
+    if (ks < 1) ks = 1;
+    if (ks > groups) ks = groups;
+    const size_t need = (size_t)KMI_GEMV_WS_HEADER + (size_t)ks * M * N * sizeof(float);
+    if (ks > 1 && (workspace == nullptr || workspace_bytes < need || (size_t)wg_x * sizeof(uint32_t) > KMI_GEMV_WS_HEADER))
+        return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: %d K splits need %zu bytes of workspace", ks, need);
+    // ring depth: what the wave's share of K can use, what vmcnt can count, what LDS holds
+    const int per_wave = (groups / ks + nw - 1) / nw;
+    if (depth <= 0 || depth > per_wave) depth = per_wave > 0 ? per_wave : 1;
+    if (depth > kn.max_depth) depth = kn.max_depth;
+    while (depth > 1 && (size_t)nw * depth * kn.slot_bytes > KMI_GEMV_RING_LDS) --depth;
+    const int mt = (M + 15) / 16;
+    size_t lds = (size_t)nw * depth * kn.slot_bytes;
+    const size_t red = (size_t)nw * mt * nt * 4 * 64 * sizeof(float);
+    if (red > lds) lds = red;
+    if (lds > KMI_GEMV_RING_LDS) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: nt=%d nw=%d needs %zu bytes of LDS", nt, nw, lds);
+    if (lds > 64 * 1024) {                                          // opt in to more than 64 KiB of dynamic LDS, once per kernel
+        static std::mutex mu;
+        static std::set<const void*> raised;
+        std::lock_guard<std::mutex> g(mu);
+        if (!raised.count(reinterpret_cast<const void*>(kn.fn))) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kn.fn), hipFuncAttributeMaxDynamicSharedMemorySize, KMI_GEMV_RING_LDS) != hipSuccess)
+                return kmi_set_error(KMI_E_LAUNCH, "kmi_gemv_w4a16: cannot raise the dynamic LDS limit");
+            raised.insert(reinterpret_cast<const void*>(kn.fn));
+        }
+    }
+    uint32_t* counters = static_cast<uint32_t*>(workspace);
+    float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + KMI_GEMV_WS_HEADER) : nullptr;
+    hipLaunchKernelGGL(kn.fn, dim3(wg_x, ks), dim3(nw * 64), lds, static_cast<hipStream_t>(stream), static_cast<half_t*>(out_f16),
+                       static_cast<const half_t*>(x_f16), static_cast<const u4_t*>(qweight),
+                       static_cast<const half_t*>(scales), static_cast<const half_t*>(scaled_zeros),
+                       static_cast<const half_t*>(bias), M, N, K, depth, partial, counters);
+    return kmi_check_launch("kmi_gemv_w4a16");
+}
+
+extern "C" int kmi_gemv_w4a16_ring_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                                       const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                                       int nt, int nw, int ks, int depth, void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = gemv_check_args(out_f16, x_f16, qweight, scales, scaled_zeros, M, N, K, G, workspace);
+    if (rc != KMI_OK) return rc;
+    return gemv_ring_launch(out_f16, x_f16, qweight, scales, scaled_zeros, bias, M, N, K, nt, nw, ks, depth, workspace,
+                            workspace_bytes, stream);
+}
+
+// What an automatic call does with a workspace of that many bytes: *form 0 = register form, 1 = ring form.
+static void gemv_plan(const void* scales, const void* scaled_zeros, int M, int N, int K, size_t workspace_bytes, bool have_ws,
+                      int* form, int* nt, int* nw, int* ks, int* depth) {
+    const int mt = (M + 15) / 16, groups = K / 128;
+    auto fits = [&](int nt_, int ks_) {                      // scratch of a split: counters of every strip + ks fp32 slices
+        const size_t need = (size_t)KMI_GEMV_WS_HEADER + (size_t)ks_ * M * N * sizeof(float);
+        const int wg_x = (N / 16 + nt_ - 1) / nt_;
+        return have_ws && workspace_bytes >= need && (size_t)wg_x * sizeof(uint32_t) <= KMI_GEMV_WS_HEADER;
+    };
+    *form = 0;
+    *depth = 0;
+    if (gemv_ring_eligible(scales, scaled_zeros, M, N, K)) {
+        bool ring = gemv_ring_default(M, N, K, true, nt, nw, ks, depth);
+        if (ring && *ks > 1 && !fits(*nt, *ks)) ring = gemv_ring_default(M, N, K, false, nt, nw, ks, depth);
+        if (ring && gemv_ring_lookup(M, *nt).fn != nullptr) {
+            *form = 1;
+            return;
+        }
+    }
+    gemv_default_cfg(M, mt, N, K, nt, nw, ks);
+    if (*ks > groups) *ks = groups;
+    if (*ks > 1 && !fits(*nt, *ks)) *ks = 1;
+    *depth = 0;
+}
+
+extern "C" int kmi_gemv_w4a16_plan(int M, int N, int K, size_t workspace_bytes, int* form, int* nt, int* nw, int* ks, int* depth) {
+    if (M < 1 || M > KMI_GEMV_MAX_M) return kmi_set_error(KMI_E_M_RANGE, "kmi_gemv_w4a16_plan: M=%d outside 1..%d", M, KMI_GEMV_MAX_M);
+    if (N <= 0 || K <= 0 || (N & 15) || (K & 127))
+        return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16_plan: need N%%16==0 and K%%128==0, got N=%d K=%d", N, K);
+    int f, a, b, c, d;
+    gemv_plan(nullptr, nullptr, M, N, K, workspace_bytes, workspace_bytes > 0, &f, &a, &b, &c, &d);
+    if (form) *form = f;
+    if (nt) *nt = a;
+    if (nw) *nw = b;
+    if (ks) *ks = c;
+    if (depth) *depth = d;
+    return KMI_OK;
+}
+
+extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* qweight, const void* scales,
+                                  const void* scaled_zeros, const void* bias, int M, int N, int K, int G,
+                                  int nt, int nw, int ks, void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = gemv_check_args(out_f16, x_f16, qweight, scales, scaled_zeros, M, N, K, G, workspace);
+    if (rc != KMI_OK) return rc;
     const int mt = (M + 15) / 16;
     const bool automatic = nt <= 0 || nw <= 0;
-    if (automatic) gemv_default_cfg(M, mt, N, K, &nt, &nw, &ks);
+    if (automatic) {
+        int form, depth;
+        gemv_plan(scales, scaled_zeros, M, N, K, workspace_bytes, workspace != nullptr, &form, &nt, &nw, &ks, &depth);
+        if (form == 1)
+            return gemv_ring_launch(out_f16, x_f16, qweight, scales, scaled_zeros, bias, M, N, K, nt, nw, ks, depth, workspace,
+                                    workspace_bytes, stream);
+    }
     if (ks < 1) ks = 1;
     gemv_fn fn = gemv_lookup(mt, nt, nw);
     if (!fn) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: no kernel for m-tiles=%d nt=%d nw=%d", mt, nt, nw);
@@ -360,6 +740,25 @@ extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* 
                        static_cast<const half_t*>(scales), static_cast<const half_t*>(scaled_zeros),
                        static_cast<const half_t*>(bias), M, N, K, partial, counters);
     return kmi_check_launch("kmi_gemv_w4a16");
+}
+
+// Arrival counters back to zero.  The kernels leave them zero themselves; this is for a buffer whose history is
+// unknown (a launch that failed or was abandoned half-way).  A plain fill kernel, so that it can be captured
+// into a graph where a memset node cannot.
+__global__ __launch_bounds__(256) void gemv_ws_reset_kernel(uint32_t* counters, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) counters[i] = 0u;
+}
+
+extern "C" int kmi_gemv_ws_reset(void* workspace, size_t workspace_bytes, void* stream) {
+    if (!workspace) return kmi_set_error(KMI_E_NULL, "kmi_gemv_ws_reset: workspace is NULL");
+    if (!kmi_aligned16(workspace)) return kmi_set_error(KMI_E_ALIGN, "kmi_gemv_ws_reset: workspace is not 16-byte aligned");
+    if (workspace_bytes < KMI_GEMV_WS_HEADER)
+        return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_ws_reset: a workspace holds at least its %d-byte counter header", KMI_GEMV_WS_HEADER);
+    const int n = KMI_GEMV_WS_HEADER / (int)sizeof(uint32_t);
+    hipLaunchKernelGGL(gemv_ws_reset_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t*>(workspace), n);
+    return kmi_check_launch("kmi_gemv_ws_reset");
 }
 
 extern "C" int kmi_gemv_w4a16(void* out_f16, const void* x_f16, const void* qweight, const void* scales,

@@ -36,6 +36,8 @@ static inline bool kmi_aligned16(const void* p) { return (reinterpret_cast<uintp
 
 #ifdef __HIPCC__
 // ---- device helpers -----------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;          // destination of a direct-to-LDS buffer load
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
 __device__ __forceinline__ h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
 __device__ __forceinline__ uint32_t as_u32(h2_t h) { return __builtin_bit_cast(uint32_t, h); }
 

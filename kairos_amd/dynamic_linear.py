@@ -20,7 +20,7 @@ import itertools
 import torch
 
 from . import ops
-from .ops import GEMV_MAX_M as _GEMV_MAX_M, _gemv_workspaces, _raw_stream
+from .ops import GEMV_MAX_M as _GEMV_MAX_M, _gemv_workspaces, _override, _raw_stream
 from .temp_cache import default_cache
 from .weight_prep import calculate_zeros_width, prepare_linear_weight
 
@@ -159,24 +159,31 @@ class DynamicLinear(torch.nn.Module):
                     and input.dtype is torch.float16 and input.is_cuda and input.is_contiguous()):
                 ptrs = self._decode_ptrs
                 if ptrs is None or ptrs[0] != self._buffers['qweight'].data_ptr():
-                    ptrs = self._decode_ptrs = self._decode_pointers(input.device)
+                    ptrs = self._decode_ptrs = self._decode_pointers()
+                if shape[-1] != ptrs[7] or input.device.index != ptrs[5]:
+                    raise ValueError(f"DynamicLinear: input of shape {tuple(shape)} on {input.device} for a layer with "
+                                     f"{ptrs[7]} input features on cuda:{ptrs[5]}")
                 out = torch.empty(shape[:-1] + (ptrs[6],), dtype=torch.float16, device=input.device)
                 st = _raw_stream(ptrs[5]) if _raw_stream is not None else ops._stream()
-                ws = _gemv_workspaces.get((ptrs[5], st))
+                ws = getattr(_override, "scratch", None)
+                ws = _gemv_workspaces.get((ptrs[5], st)) if ws is None else ws.gemv
                 if ws is None:
                     ws = ops.gemv_workspace_for(input.device, st)
                 rc = ptrs[4](out.data_ptr(), input.data_ptr(), ptrs[0], ptrs[1], ptrs[2], ptrs[3], m, ptrs[6], ptrs[7], ptrs[8],
                              ws.data_ptr(), ws.numel(), st)
                 if rc < 0:
+                    if rc == -6:               # the runtime rejected the launch: leave the counters in a known state
+                        ops._lib.load().kmi_gemv_ws_reset(ws.data_ptr(), ws.numel(), st)
                     ops._lib.check(rc)
                 return out
         return self._forward_any(input)
 
-    def _decode_pointers(self, device):
+    def _decode_pointers(self):
         N, K = self.shape
+        dev = self.qweight.device
         return (self.qweight.data_ptr(), self.scales.data_ptr(), self.scaled_zeros.data_ptr(),
-                0 if self.bias is None else self.bias.data_ptr(), ops._lib.load().kmi_gemv_w4a16, device.index or 0,
-                N, K, self.group_size)
+                0 if self.bias is None else self.bias.data_ptr(), ops._lib.load().kmi_gemv_w4a16,
+                dev.index if dev.index is not None else torch.cuda.current_device(), N, K, self.group_size)
 
     @torch.no_grad()
     def _forward_any(self, input) -> torch.Tensor:

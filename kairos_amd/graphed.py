@@ -9,8 +9,12 @@ exactly as serving stacks do with CUDA graphs.
 Capture rules this module enforces or relies on:
   * every kernel of the library launches on torch's current stream, so torch's stream capture records it;
   * the library records no memset nodes (none of its entry points clears memory);
-  * the temp cache and the capture stream's split-K scratch are created BEFORE capture, by warm-up calls on that
-    stream (they must not come from the graph's private pool: the temp cache is shared with eager calls);
+  * the temp cache is created BEFORE capture, by warm-up calls on the capture stream (it must not come from the
+    graph's private pool: it is shared with eager calls);
+  * the split-K and small-M scratch of the captured kernels belongs to the GraphedCallable (an ops.Scratch made or
+    given at construction), not to a stream: a replay runs on whatever stream is current, so scratch looked up by
+    the capture stream's handle could be in use by eager work, or by another graph, on a different stream at that
+    moment.  Replays of ONE instance, and of instances that share a Scratch, must be ordered on one stream;
   * the temp cache is invalidated right before capture, so every conversion the step needs is part of the
     graph, and after every replay, because the graph rewrites the cache behind the host-side tag's back;
   * inputs are copied into static buffers before each replay; outputs are the static tensors captured.
@@ -29,16 +33,20 @@ class GraphedCallable:
     before the next call.
     """
 
-    def __init__(self, fn, example_inputs, warmup=3, caches=None):
-        """caches: the TempCache objects the captured modules use (default: the process-wide one)."""
+    def __init__(self, fn, example_inputs, warmup=3, caches=None, scratch=None):
+        """caches: the TempCache objects the captured modules use (default: the process-wide one).  scratch: the
+        ops.Scratch whose buffers the captured kernels use (default: a new one, 96 MiB, owned by this instance);
+        pass one Scratch to several instances whose replays are ordered on one stream (e.g. the batch buckets of
+        one decode loop) to share it."""
         if not torch.cuda.is_available():
             raise RuntimeError("GraphedCallable: needs a GPU")
         self._static_in = [x.clone() for x in example_inputs]
+        self.scratch = scratch if scratch is not None else ops.Scratch(self._static_in[0].device)
         side = torch.cuda.Stream()                      # default priority; warm-up AND capture run on it
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(warmup):                     # sizes the temp cache, settles the LUT memo, creates this
-                fn(*self._static_in)                    # stream's split-K scratch outside the graph's memory pool
+        with torch.cuda.stream(side), self.scratch:
+            for _ in range(warmup):                     # sizes the temp cache and settles the LUT memo
+                fn(*self._static_in)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self._caches = list(caches) if caches is not None else [default_cache()]
@@ -46,7 +54,7 @@ class GraphedCallable:
         for c in self._caches:
             c.prepare_for_capture(self._static_in[0].device)
         self._graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self._graph, stream=side):
+        with self.scratch, torch.cuda.graph(self._graph, stream=side):
             self._static_out = fn(*self._static_in)
         self._invalidate()
         self.replays = 0
@@ -83,11 +91,11 @@ class GraphedCallable:
         return self._static_in
 
 
-def graph_layer(linears, example_input_for):
+def graph_layer(linears, example_input_for, scratch=None):
     """Convenience: one graph over `[lin(x) for lin in linears]`, `example_input_for(lin)` giving each input."""
     xs = [example_input_for(l) for l in linears]
 
     def step(*inputs):
         return tuple(l(x) for l, x in zip(linears, inputs))
 
-    return GraphedCallable(step, xs)
+    return GraphedCallable(step, xs, scratch=scratch)

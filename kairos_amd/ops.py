@@ -4,6 +4,8 @@ replace (kernels/csrc/pybind.cpp:18-24, thirdparty/AWQ/kernels/csrc/pybind.cpp:2
 PyTorch only supplies device memory and the current stream; every computation happens in
 libkairos_mi.so.  Outputs are allocated by the caller unless the reference function returns one.
 """
+import threading
+
 import torch
 
 from . import _lib
@@ -202,68 +204,159 @@ def _flat2d(x):
     return x.reshape(-1, x.shape[-1])
 
 
-def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZE, bias=None, cfg=None):
-    """W4A16 for small m (gemv_cuda.cu:245-463).  Returns fp16 [*x.shape[:-1], n].  cfg: (column tiles per wave, waves
-    per workgroup[, workgroups over K]) for tuning; None = the library's choice."""
+def gemv_forward(x, qweight, scales, scaled_zeros, m, n, k, group_size=GROUP_SIZE, bias=None, cfg=None, ring=None):
+    """W4A16 for small m (gemv_cuda.cu:245-463).  Returns fp16 [*x.shape[:-1], n].  Tuning: cfg = (column tiles per wave,
+    waves per workgroup[, workgroups over K]) runs the register form, ring = (column tiles, waves, workgroups over K,
+    ring depth) the ring form; neither = the library's choice."""
     _need(x, torch.float16, "x"); _need(qweight, torch.int16, "qweight")
+    if x.shape[-1] != k or x.numel() != m * k:
+        raise ValueError(f"gemv_forward: x of shape {tuple(x.shape)} is not {m} rows of {k}")
+    if qweight.shape[0] * 4 != n or qweight.shape[1] != k:
+        raise ValueError(f"gemv_forward: packed weight {tuple(qweight.shape)} does not hold {n} x {k}")
     out = torch.empty(x.shape[:-1] + (n,), dtype=torch.float16, device=x.device)
     lib = _lib.load()
-    nt, nw, ks = (tuple(cfg) + (1,))[:3] if cfg is not None else (0, 0, 0)
     st = _stream()
     ws = gemv_workspace_for(x.device, st)
-    _call("gemv_w4a16", m, n, k, lib.kmi_gemv_w4a16_cfg, out.data_ptr(), x.data_ptr(), qweight.data_ptr(),
-          scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, ks, ws.data_ptr(),
-          ws.numel(), st)
+    try:
+        if ring is not None:
+            nt, nw, ks, depth = ring
+            _call("gemv_w4a16", m, n, k, lib.kmi_gemv_w4a16_ring_cfg, out.data_ptr(), x.data_ptr(), qweight.data_ptr(),
+                  scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, ks, depth,
+                  ws.data_ptr(), ws.numel(), st)
+        else:
+            nt, nw, ks = (tuple(cfg) + (1,))[:3] if cfg is not None else (0, 0, 0)
+            _call("gemv_w4a16", m, n, k, lib.kmi_gemv_w4a16_cfg, out.data_ptr(), x.data_ptr(), qweight.data_ptr(),
+                  scales.data_ptr(), scaled_zeros.data_ptr(), _ptr(bias), m, n, k, group_size, nt, nw, ks, ws.data_ptr(),
+                  ws.numel(), st)
+    except _lib.KairosMiError as e:
+        if e.code == -6:                   # the runtime rejected a launch: leave the counters in a known state
+            lib.kmi_gemv_ws_reset(ws.data_ptr(), ws.numel(), st)
+        raise
     return out
 
 
 WORKSPACE_BYTES = 64 << 20
-_workspaces = {}                 # (device index, raw stream handle) -> uint8 tensor; never resized, never shared
+GEMV_WORKSPACE_BYTES = 65536 + (32 << 20)      # arrival counters (KMI_GEMV_WS_HEADER) + fp32 partial sums
+_workspaces = {}                 # (device index, raw stream handle) -> uint8 tensor; never resized
+_gemv_workspaces = {}            # the same for the small-M kernel's scratch (zeroed counter header first)
+_override = threading.local()    # .scratch: a Scratch that replaces the per-stream buffers in this thread, or None
+
+
+class Scratch:
+    """One owner's pair of scratch buffers: split-K partial sums of the GEMMs (`gemm`) and the small-M kernel's
+    arrival counters + partial sums (`gemv`, counters zeroed here).  Work that shares a Scratch must be ordered (one
+    stream, or replays that wait for each other): two launches using it at the same time race on the partial sums.
+    `with scratch:` makes every call of this thread use it instead of the per-stream buffers -- a graph captured inside
+    the block owns its scratch, whatever stream it is replayed on."""
+
+    def __init__(self, device="cuda"):
+        dev = torch.device(device)
+        idx = dev.index if dev.index is not None else torch.cuda.current_device()
+        self.device_index = idx
+        self.gemm = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+        self.gemv = torch.zeros(GEMV_WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+
+    def __enter__(self):
+        self._prev = getattr(_override, "scratch", None)
+        _override.scratch = self
+        return self
+
+    def __exit__(self, *exc):
+        _override.scratch = self._prev
+        return False
+
+    def reset(self):
+        """Arrival counters back to zero (after a call on this scratch that did not run to completion)."""
+        _lib.check(_lib.load().kmi_gemv_ws_reset(self.gemv.data_ptr(), self.gemv.numel(), _stream()))
+
+
+def _index_of(device):
+    dev = torch.device(device)
+    return dev.index if dev.index is not None else torch.cuda.current_device()
+
+
+def _new_scratch(idx, nbytes, zero, what):
+    # Allocating under stream capture would take the buffer from the graph's private pool (and, zeroed, record a
+    # memset node) and then hand it to eager calls as well: refuse, and say what to do instead.
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(f"the {what} scratch of this stream does not exist yet and cannot be created during graph "
+                           "capture: call kairos_amd.ops.ensure_workspace(device, stream) before capturing, or capture "
+                           "inside `with kairos_amd.ops.Scratch(device):`")
+    make = torch.zeros if zero else torch.empty
+    return make(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
 
 
 def workspace_for(device, stream=None):
-    """Split-K scratch of the calling stream: one fixed-size buffer per (device, stream), created on first use and
-    handed to every GEMM call as (pointer, bytes).  Two streams never share one, so concurrent GEMMs cannot race on
-    the partial sums; the size never changes, so a pointer baked into a captured graph stays valid for the life of
-    the process (drop_workspaces() is for tests only)."""
-    dev = torch.device(device)
-    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    """Split-K scratch for a GEMM call: the active Scratch of this thread if there is one, else one fixed-size buffer
+    per (device, stream), created on first use.  Streams are told apart by their raw handle; a handle that the runtime
+    hands out again after its stream was destroyed finds the old buffer, which is harmless as long as the destroyed
+    stream's work has finished.  A pointer baked into a captured graph stays valid until release_workspace /
+    drop_workspaces; a graph that must not share scratch with eager work on the same stream captures under a Scratch."""
+    ov = getattr(_override, "scratch", None)
+    if ov is not None:
+        return ov.gemm
+    idx = _index_of(device)
     if stream is None:
         stream = _stream()
     ws = _workspaces.get((idx, stream))
     if ws is None:
-        ws = _workspaces[(idx, stream)] = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+        ws = _workspaces[(idx, stream)] = _new_scratch(idx, WORKSPACE_BYTES, False, "split-K")
     return ws
 
 
-GEMV_WORKSPACE_BYTES = 65536 + (32 << 20)      # arrival counters (KMI_GEMV_WS_HEADER) + fp32 partial sums
-_gemv_workspaces = {}
-
-
 def gemv_workspace_for(device, stream=None):
-    """Scratch of the small-M kernel's split over K, per (device, stream) like workspace_for, but ZEROED at creation:
-    its first 64 KiB are arrival counters that the kernels return to zero themselves.  Kept apart from the GEMM
-    scratch, whose partial sums would overwrite the counters."""
-    dev = torch.device(device)
-    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    """Scratch of the small-M kernel's split over K, chosen like workspace_for, but ZEROED at creation: its first 64 KiB
+    are arrival counters that the kernels return to zero themselves.  Kept apart from the GEMM scratch, whose partial
+    sums would overwrite the counters."""
+    ov = getattr(_override, "scratch", None)
+    if ov is not None:
+        return ov.gemv
+    idx = _index_of(device)
     if stream is None:
         stream = _stream()
     ws = _gemv_workspaces.get((idx, stream))
     if ws is None:
-        ws = _gemv_workspaces[(idx, stream)] = torch.zeros(GEMV_WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+        ws = _gemv_workspaces[(idx, stream)] = _new_scratch(idx, GEMV_WORKSPACE_BYTES, True, "small-M")
     return ws
 
 
+def gemv_workspace_reset(device="cuda", stream=None):
+    """Zeroes the arrival counters of the calling (or given) stream's small-M scratch with a small kernel: after a
+    call that raised, or whenever the buffer's history is in doubt."""
+    ws = gemv_workspace_for(device, stream)
+    _lib.check(_lib.load().kmi_gemv_ws_reset(ws.data_ptr(), ws.numel(), _stream() if stream is None else stream))
+
+
 def ensure_workspace(device="cuda", stream=None):
-    """Creates the calling (or given) stream's split-K scratch ahead of time, e.g. before a graph capture on it."""
+    """Creates the calling (or given) stream's scratch buffers ahead of time, e.g. before a graph capture on it."""
     gemv_workspace_for(device, stream)
     return workspace_for(device, stream)
 
 
+def release_workspace(device="cuda", stream=None):
+    """Forgets the scratch of one (device, stream); the memory returns to the allocator once no tensor refers to it.
+    Not while work that uses it is pending or a captured graph that used it is alive."""
+    idx = _index_of(device)
+    if stream is None:
+        stream = _stream()
+    _workspaces.pop((idx, stream), None)
+    _gemv_workspaces.pop((idx, stream), None)
+
+
 def drop_workspaces():
-    """Forgets every scratch buffer (tests).  Not while a captured graph that used one is still alive."""
+    """Forgets every per-stream scratch buffer (tests).  Not while a captured graph that used one is still alive."""
     _workspaces.clear()
     _gemv_workspaces.clear()
+
+
+def gemv_plan(M, N, K, workspace_bytes=GEMV_WORKSPACE_BYTES):
+    """What the small-M entry point does for this shape (host only): dict with form ('register' / 'ring'), nt (16-column
+    tiles per wave), nw (waves per workgroup), ks (workgroups sharing a strip's K range), depth (ring slots asked for)."""
+    import ctypes
+    v = [ctypes.c_int(0) for _ in range(5)]
+    _lib.check(_lib.load().kmi_gemv_w4a16_plan(int(M), int(N), int(K), int(workspace_bytes), *[ctypes.byref(c) for c in v]))
+    return {"form": "ring" if v[0].value == 1 else "register", "nt": v[1].value, "nw": v[2].value, "ks": v[3].value,
+            "depth": v[4].value}
 
 
 def gemm_splits_for(lane, M, N, K, workspace_bytes=WORKSPACE_BYTES):

@@ -45,6 +45,12 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 65, 64, 128, 128, None, 0, None) == -4
     assert lib.kmi_gemv_w4a16(16, 16, 16, 16, 16, None, 4, 60, 128, 128, None, 0, None) == -2
     assert lib.kmi_gemv_w4a16_cfg(16, 16, 16, 16, 16, None, 4, 64, 1024, 128, 1, 8, 2, None, 0, None) == -2   # a forced K split needs scratch
+    assert lib.kmi_gemv_w4a16_ring_cfg(16, 16, 16, 16, 16, None, 4, 64, 1024, 128, 1, 8, 2, 2, None, 0, None) == -2   # the same for the ring form
+    assert lib.kmi_gemv_w4a16_ring_cfg(16, 16, 16, 16, 16, None, 4, 64, 1024, 128, 1, 3, 1, 2, None, 0, None) == -2   # 1, 2, 4 or 8 waves
+    assert lib.kmi_gemv_w4a16_ring_cfg(16, 16, 16, 18, 16, None, 4, 64, 1024, 128, 1, 8, 1, 2, None, 0, None) == -5   # tables: 4-byte aligned
+    assert lib.kmi_gemv_w4a16_ring_cfg(16, 16, 16, 16, 16, None, 40, 64, 1024, 128, 4, 8, 1, 2, None, 0, None) == -2  # 3 x 4 accumulator tiles
+    assert lib.kmi_gemv_ws_reset(None, 1 << 20, None) == -1 and lib.kmi_gemv_ws_reset(16, 1024, None) == -2
+    assert lib.kmi_gemv_ws_reset(24, 1 << 20, None) == -5
     assert lib.kmi_gemm_w8a8(16, 16, 16, 16, 16, None, 4, 64, 100, None, 0, None) == -2
     assert lib.kmi_gemm_w8a8(16, 16, 16, None, 16, None, 4, 64, 128, None, 0, None) == -1
     assert lib.kmi_quant_act_i8(16, 16, 16, 4, 12, None) == -2
@@ -138,3 +144,39 @@ def test_lut_matches_oracle_on_reference_tables(lib, golden_dir):
             for m in list(range(1, 2500)) + [5, 5, 30720, 30721, 10 ** 6, 1, 1]:
                 assert lib.kmi_lut_get(h, m) == mine.get(m)
             lib.kmi_lut_free(h)
+
+
+def test_small_m_plan_is_host_logic(lib):
+    """Which form and split the small-M entry point takes (measured rule, see the kernel file): the ring form beyond 16
+    rows everywhere and from 8 rows (1 where K is long) on narrow weights, the register form on wide weights up to 16
+    rows; long, narrow weights split K over workgroups only when the caller brought scratch for it."""
+    import ctypes
+    from kairos_amd import ops
+
+    def plan(M, N, K, ws=ops.GEMV_WORKSPACE_BYTES):
+        return ops.gemv_plan(M, N, K, ws)
+
+    assert plan(1, 28672, 4096)["form"] == "register" and plan(16, 28672, 4096)["form"] == "register"
+    assert plan(32, 28672, 4096) == {"form": "ring", "nt": 4, "nw": 8, "ks": 1, "depth": 2}
+    assert plan(1, 4096, 4096)["form"] == "register" and plan(8, 4096, 4096)["form"] == "ring"
+    assert plan(16, 6144, 4096)["form"] == "register" and plan(32, 6144, 4096)["nt"] == 2
+    assert plan(1, 4096, 14336) == {"form": "ring", "nt": 1, "nw": 8, "ks": 1, "depth": 2}
+    assert plan(16, 4096, 14336) == {"form": "ring", "nt": 2, "nw": 8, "ks": 2, "depth": 2}
+    assert plan(16, 4096, 14336, 0)["ks"] == 1 and plan(16, 4096, 14336, 0)["form"] == "ring"      # no scratch, no split
+    assert plan(32, 8192, 28672) == {"form": "ring", "nt": 4, "nw": 8, "ks": 2, "depth": 2}
+    assert plan(64, 57344, 8192) == {"form": "ring", "nt": 2, "nw": 8, "ks": 1, "depth": 2}
+    assert plan(4, 4096, 14336 * 2, 1 << 16)["ks"] == 1                                              # scratch too small for a split
+    z = ctypes.c_int(0)
+    assert lib.kmi_gemv_w4a16_plan(0, 4096, 4096, 0, None, None, None, None, None) == -4
+    assert lib.kmi_gemv_w4a16_plan(4, 4090, 4096, 0, ctypes.byref(z), None, None, None, None) == -2
+    assert lib.kmi_gemv_w4a16_plan(4, 4096, 4096, 0, None, None, None, None, None) == 0              # outputs are optional
+
+
+def test_tile_queries_survive_empty_products(lib):
+    """The host queries run before the entry points' own M == 0 early return (a tracer asks them): no division by the
+    tile count of an empty product."""
+    for M, N, K in ((0, 4096, 4096), (4096, 0, 4096), (-3, 4096, 4096)):
+        assert lib.kmi_gemm_w4a8_pick_tile(M, N, K) in (128, 130, 192, 256, 448, 512, 640)
+        assert lib.kmi_gemm_pick_tile(M, N, K) in (64, 128, 192, 256, 320)
+        assert lib.kmi_gemm_w4a16_wp_rows(M, N, K) in (0, 32, 64, 128)
+    assert lib.kmi_gemm_w4a8_pick_tile(16, 4096, 0) == 128

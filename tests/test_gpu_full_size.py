@@ -103,6 +103,43 @@ def test_gemv_periodic_weights_70b_shapes(ops, N, K):
         assert O.max_abs_rel(first.cpu().numpy(), ref) < 1e-2
 
 
+@pytest.mark.parametrize("N,K", [(6144, 4096), (28672, 4096), (4096, 14336), (4096, 4096)])
+def test_gemv_automatic_choice_8b_shapes_against_oracle(ops, N, K):
+    """The small-M entry point as the benchmark calls it (no tuning arguments) at the true Llama-3-8B shapes, on the
+    benchmark's kind of data, against the oracle on 1024 sampled columns (columns are independent of each other); the
+    plan query must report the launch that ran: a K split over workgroups on the long, narrow down projection, the ring
+    form wherever the library's rule says so."""
+    w = O.synth_weights(N, K, seed=10)
+    p = ops.prepare_weight(dev(w))
+    blocks = np.sort(np.random.default_rng(N + K).choice(N // 16, size=64, replace=False))     # 64 strips of 16 columns
+    cols = (blocks[:, None] * 16 + np.arange(16)[None, :]).reshape(-1)
+    q_rows = (blocks[:, None] * 4 + np.arange(4)[None, :]).reshape(-1)                          # packed rows of those strips
+    cidx = torch.from_numpy(cols).cuda()
+    qs = p["qweight"][torch.from_numpy(q_rows).cuda()].cpu().numpy()
+    sc, sz = p["scales"][:, cidx].cpu().numpy(), p["scaled_zeros"][:, cidx].cpu().numpy()
+    w16_ref = O.dequant_to_f16(qs, sc, sz)
+    seen = set()
+    for M in (1, 8, 16, 32):
+        plan = ops.gemv_plan(M, N, K)
+        seen.add((plan["form"], plan["ks"] > 1))
+        x = O.synth_acts(M, K, seed=M)
+        out = ops.gemv_forward(dev(x), p["qweight"], p["scales"], p["scaled_zeros"], M, N, K, 128)
+        torch.cuda.synchronize()
+        assert O.max_abs_rel(out[:, cidx].cpu().numpy(), O.gemm_f16(x, w16_ref)) < 2e-3, (M, plan)
+        if plan["form"] == "register":      # the tuning entry point with the planned split is the same launch
+            same = ops.gemv_forward(dev(x), p["qweight"], p["scales"], p["scaled_zeros"], M, N, K, 128, cfg=(plan["nt"], plan["nw"], plan["ks"]))
+        else:
+            same = ops.gemv_forward(dev(x), p["qweight"], p["scales"], p["scaled_zeros"], M, N, K, 128,
+                                    ring=(plan["nt"], plan["nw"], plan["ks"], plan["depth"]))
+        assert torch.equal(same.view(torch.int16), out.view(torch.int16)), (M, plan)
+    if (N, K) == (4096, 14336):
+        assert any(split for _, split in seen), seen           # the split over workgroups engaged on this shape
+    if (N, K) == (28672, 4096):
+        assert ("register", False) in seen and any(form == "ring" for form, _ in seen), seen
+    ws = ops.gemv_workspace_for("cuda")
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0
+
+
 @pytest.mark.parametrize("N,K", [(28672, 4096), (4096, 14336), (37888, 3584)])
 def test_conversion_layouts_agree_full_size(ops, N, K):
     """Conversion at full size: with s = 1, z = 0 the fp16 result is the unpacked nibble itself (pure layout), the int8

@@ -236,6 +236,72 @@ def test_gemv_bias_and_ragged_strip(ops):
     assert O.max_abs_rel(host(out), ref) < 2e-3
 
 
+# ---- ring form of the small-M kernel (operands travel global -> LDS, per-wave ring of slots)
+@pytest.mark.parametrize("M,nt,nw,ks", [(1, 1, 8, 1), (3, 2, 4, 1), (4, 7, 8, 1), (5, 2, 8, 2), (8, 8, 4, 1), (9, 3, 8, 1),
+                                          (16, 4, 8, 4), (17, 1, 8, 1), (32, 4, 8, 2), (33, 2, 4, 1), (48, 2, 8, 1), (64, 2, 4, 3)])
+def test_gemv_ring_equals_register_form(ops, M, nt, nw, ks):
+    """Same lanes, same arithmetic, same summation order as the register form with the same split: the two forms agree
+    bit for bit at every ring depth (1 = load, wait, compute; 0 = as deep as fits), with bias and a ragged last strip."""
+    N, K = 336, 3584                                         # 21 strips (ragged for nt = 2, 4, 8), 28 groups
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=60 + M)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float16)
+    ref = (O.gemm_w4a16(x, p["qweight"], p["scales"], p["scaled_zeros"]).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    args = (dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+    want = ops.gemv_forward(*args, bias=dev(bias), cfg=(nt, nw, ks))
+    assert O.max_abs_rel(host(want), ref) < 2e-3
+    for depth in (1, 2, 3, 0):
+        got = ops.gemv_forward(*args, bias=dev(bias), ring=(nt, nw, ks, depth))
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), depth
+    ws = ops.gemv_workspace_for("cuda")
+    torch.cuda.synchronize()
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0          # arrival counters left at zero
+
+
+@pytest.mark.parametrize("nw", [1, 2, 8])
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 8, 12, 16, 24, 32, 40, 48, 56, 64])
+def test_gemv_ring_every_row_count(ops, M, nw):
+    """Every activation-load count of the ring form (1, 2, 4, 8, 12, 16 loads per group) against the oracle, also with
+    fewer K groups than ring slots and with waves that get no group at all (K = 512: four groups, eight waves)."""
+    N = 256
+    for K in (512, 2048):
+        p = prep(N, K)
+        x = O.synth_acts(M, K, seed=M)
+        nt = 2 if M <= 32 else 1
+        out = ops.gemv_forward(dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128, ring=(nt, nw, 1, 0))
+        assert O.max_abs_rel(host(out), O.gemm_f16(x, p["w16"])) < 2e-3, K
+
+
+def test_gemv_ring_refuses_what_it_cannot_run(ops):
+    from kairos_amd._lib import KairosMiError
+    N, K, M = 256, 512, 20
+    p = prep(N, K)
+    args = (dev(O.synth_acts(M, K, seed=1)), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+    with pytest.raises(KairosMiError):
+        ops.gemv_forward(*args, ring=(5, 8, 1, 2))            # two row tiles x five column tiles: too many accumulators
+    with pytest.raises(KairosMiError):
+        ops.gemv_forward(*args, ring=(2, 3, 1, 2))            # waves per workgroup: 1, 2, 4 or 8
+    with pytest.raises(ValueError):
+        ops.gemv_forward(dev(O.synth_acts(M, 256, seed=1)), *args[1:])     # activation rows shorter than K
+
+
+def test_gemv_workspace_reset(ops):
+    """Counters of unknown history: the reset kernel zeroes the header and nothing else; a split call works afterwards."""
+    N, K, M = 320, 3584, 8
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=2)
+    args = (dev(x), dev(p["qweight"]), dev(p["scales"]), dev(p["scaled_zeros"]), M, N, K, 128)
+    want = ops.gemv_forward(*args, cfg=(2, 8, 4))
+    ws = ops.gemv_workspace_for("cuda")
+    ws[:65536] = 7                                            # as a launch that died half-way might leave them
+    ws[65536:65536 + 64] = 9
+    ops.gemv_workspace_reset("cuda")
+    torch.cuda.synchronize()
+    assert int(ws[:65536].view(torch.int32).abs().sum().item()) == 0 and int(ws[65536:65536 + 64].min().item()) == 9
+    assert torch.equal(ops.gemv_forward(*args, cfg=(2, 8, 4)).view(torch.int16), want.view(torch.int16))
+    assert torch.equal(ops.gemv_forward(*args, ring=(2, 8, 4, 2)).view(torch.int16), want.view(torch.int16))
+
+
 # ------------------------------------------------------------------ MFMA GEMMs
 GEMM_M = [1, 7, 64, 65, 130, 300]
 
