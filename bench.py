@@ -138,11 +138,16 @@ class Tracer:
         return agg
 
 
+CPU_M_SUBSET = (1, 16, 256, 1024, 4096)          # the M over which the CPU leg's `value` is averaged
+
+
 def cpu_baseline(gpu_us_per_layer_by_m):
     """The oracle's W4A16 lane (unpack, fp16 FMA dequantisation, fp32-accumulated matmul) for the four linears of the
-    layer, on the host cores of this box: the same unit as `value`, comparable with the per-M table.  The oracle's own
-    functions run on column slabs of the weight, one slab per worker thread (numpy releases the interpreter lock
-    inside its loops); BLAS is held to one thread per worker.  Also timed on a single thread."""
+    layer, on the host cores of this box.  `value` is microseconds per layer averaged over CPU_M_SUBSET -- the unit of the
+    headline `value`, on a stated subset of its M grid so that the leg stays bounded; the M = 16 figure (the case the
+    reference can run on a CPU) is kept beside it.  The oracle's own functions run on column slabs of the weight, one
+    slab per worker thread (numpy releases the interpreter lock inside its loops); BLAS is held to one thread per
+    worker.  Also timed on a single thread at M = 16."""
     import numpy as np
     from concurrent.futures import ThreadPoolExecutor
     from oracle import kairos_oracle as O
@@ -162,7 +167,7 @@ def cpu_baseline(gpu_us_per_layer_by_m):
         sc = (rng.random((gp, N), dtype=np.float32) * 0.01 + 0.002).astype(np.float16)
         sz = (-(sc.astype(np.float32) * 7.5)).astype(np.float16)
         weights.append((N, K, qw, sc, sz))
-    acts = {(M, K): O.synth_acts(M, K) for M in (16, 1024) for K in sorted({k for _, _, k in LAYER})}
+    acts = {(M, K): O.synth_acts(M, K) for M in CPU_M_SUBSET for K in sorted({k for _, _, k in LAYER})}
     SLAB = 256                                               # weight rows per task (a multiple of the 4-row interleave)
 
     def layer(M, pool):
@@ -175,30 +180,38 @@ def cpu_baseline(gpu_us_per_layer_by_m):
             assert sum(p.shape[1] for p in parts) == N
         return time.perf_counter() - t0
 
-    def median_of(M, pool, passes):
-        layer(M, pool)
+    def median_of(M, pool, passes, warm=True):
+        if warm:
+            layer(M, pool)
         ts = sorted(layer(M, pool) for _ in range(passes))
         return ts[len(ts) // 2], sum(ts)
 
     ctx = threadpool_limits(limits=1) if threadpool_limits else None
     if ctx:
         ctx.__enter__()
+    t_all = time.perf_counter()
     try:
         with ThreadPoolExecutor(max_workers=cores) as pool:
-            m16, w16 = median_of(16, pool, 7)
-            m1k, w1k = median_of(1024, pool, 3)
-        one, w1 = median_of(16, None, 3)
+            per_m = {}
+            for M in CPU_M_SUBSET:
+                passes = 7 if M <= 16 else 3 if M <= 1024 else 1
+                per_m[M] = median_of(M, pool, passes, warm=M <= 1024)[0]
+        one, _w1 = median_of(16, None, 3)
     finally:
         if ctx:
             ctx.__exit__(None, None, None)
-    return {"value": m16 * 1e6, "unit": "us/layer at M=16 (W4A16 lane)", "cores": cores, "kind": "port",
-            "by_m_us_per_layer": {"16": round(m16 * 1e6), "1024": round(m1k * 1e6)},
-            "one_thread_us_per_layer_m16": round(one * 1e6),
+    spent = time.perf_counter() - t_all
+    mean_us = sum(per_m.values()) / len(per_m) * 1e6
+    gpu_mean = sum(gpu_us_per_layer_by_m[M] for M in CPU_M_SUBSET) / len(CPU_M_SUBSET)
+    return {"value": round(mean_us, 1), "unit": f"us/layer (mean over M in {list(CPU_M_SUBSET)}, W4A16 lane)", "cores": cores,
+            "kind": "port", "by_m_us_per_layer": {str(M): round(t * 1e6) for M, t in per_m.items()},
+            "m16_us_per_layer": round(per_m[16] * 1e6), "one_thread_us_per_layer_m16": round(one * 1e6),
+            "gpu_us_per_layer_same_m_subset": round(gpu_mean, 2),
             "sample": f"numpy oracle (unpack, fp16-FMA dequantise, fp32 matmul) of the layer's four linears on {cores} "
-                      f"worker threads over {SLAB}-row weight slabs: M=16 median of 7 passes {m16 * 1e3:.0f} ms, M=1024 "
-                      f"median of 3 passes {m1k * 1e3:.0f} ms; one thread at M=16 {one * 1e3:.0f} ms "
-                      f"(about {w16 + w1k + w1 + m16 + m1k + one:.0f} s of wall time in all); the GPU spends "
-                      f"{gpu_us_per_layer_by_m[16]:.1f} us at M=16 and {gpu_us_per_layer_by_m[1024]:.1f} us at M=1024 on the same layer"}
+                      f"worker threads over {SLAB}-row weight slabs, M in {list(CPU_M_SUBSET)}: medians of 7 / 7 / 3 / 3 / 1 passes "
+                      + ", ".join(f"M={M} {t * 1e3:.0f} ms" for M, t in per_m.items())
+                      + f"; one thread at M=16 {one * 1e3:.0f} ms (about {spent:.0f} s of wall time in all); the GPU spends "
+                      f"{gpu_mean:.1f} us per layer on the same M subset ({gpu_us_per_layer_by_m[16]:.1f} us at M=16)"}
 
 
 def main():
@@ -210,6 +223,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-lane sweep table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the small-M layers")
+    ap.add_argument("--no-oracle", action="store_true", help="skip the keep-everything-resident (SwitchLinear) comparison")
     ap.add_argument("--dump-launches", default=None, help="write every event-bracketed launch of the replay (JSON)")
     ap.add_argument("--resident-cache-mb", type=int, default=0,
                     help="keep converted weights in an LRU cache of this many MiB (0 = the single shared temp buffer, "
@@ -365,6 +379,8 @@ def main():
                 "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
                 "launches": dom["launches"], "avg_launch_us": round(avg_dur * 1e6, 2),
                 "share_of_kernel_time": round(dom["sec"] / total_kernel_sec, 4)}
+    # every label together: time the step's launches would take at their rooflines over the time they took
+    roofline_all = round(sum(a["ideal_sec"] for a in agg.values()) / total_kernel_sec, 4)
     kernels = {k: {"launches": a["launches"], "avg_us": round(a["sec"] / a["launches"] * 1e6, 2),
                    "share": round(a["sec"] / total_kernel_sec, 4),
                    "roofline_frac": round(a["ideal_sec"] / a["sec"], 4)} for k, a in sorted(agg.items())}
@@ -408,6 +424,85 @@ def main():
             g = GraphedCallable(graph_step, xs)
             graph_by_m[M] = round(time_calls(lambda i=0: g.replay(), 20) / args.copies, 2)
             del g
+
+    # ---- the reference's own yardstick: the keep-everything-resident layer ("Oracle", kairos/switch_linear.py:43-213,
+    # README.md:120-123: the switched single-copy layer reaches 93 % of it at +5 % memory on an A100).  Every format of
+    # every weight stays in HBM (no lane converts), each (shape, M) runs the lane that measures fastest here, and the
+    # same 13-M step is timed the same way.  Outside the timed region of `value`.
+    keep_all = None
+    if not args.no_oracle:
+        from kairos_amd.switch_linear import SwitchLinear
+        o_layers = []
+        for li, (_name, N, K) in enumerate(LAYER):
+            row = []
+            for c in range(args.copies):
+                sl = SwitchLinear(K, N, False, dev, 128)
+                for key in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1"):
+                    setattr(sl, key, getattr(layers[li][c], key))           # the very weights of the switched layers
+                sl._ensure_resident()
+                row.append(sl)
+            o_layers.append(row)
+        torch.cuda.synchronize()
+        o_prof = Profiler(shapes)
+        o_lanes = ["w4a16_gemv", "w4a16_gemm", "w8a8", "w4a8_qserve", "fp16"]
+        o_pick = {}
+        for li, (lname, N, K) in enumerate(LAYER):
+            for M in M_GRID:
+                best = None
+                for lane in o_lanes:
+                    if lane == "w4a16_gemv" and M > ops.GEMV_MAX_M:
+                        continue
+                    cid = COMP_TYPE_NAME[lane]
+                    us = time_calls(lambda i=0, cid=cid, M=M, K=K, li=li: o_layers[li][i % args.copies]._forward(acts[(M, K)], M, cid),
+                                    20 if M <= 512 else 6)
+                    if best is None or us < best[0]:
+                        best = (us, lane)
+                o_pick[(lname, M)] = best[1]
+                o_prof.record_best_comp((N, K), M, best[1])
+        SwitchLinear.prof = o_prof
+
+        def o_step(s):
+            for mi, M in enumerate(M_GRID):
+                c = (s * len(M_GRID) + mi) % args.copies
+                for li, (_n, _N, K) in enumerate(LAYER):
+                    o_layers[li][c](acts[(M, K)])
+        for s in range(args.warmup):
+            o_step(s)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for s in range(args.steps):
+            o_step(s)
+        b.record()
+        torch.cuda.synchronize()
+        o_us = a.elapsed_time(b) * 1e3 / args.steps / len(M_GRID)
+        o_by_m = {}
+        for M in M_GRID:
+            def o_call(i=0, M=M):
+                for li, (_n, _N, K) in enumerate(LAYER):
+                    o_layers[li][i % args.copies](acts[(M, K)])
+            o_by_m[M] = round(time_calls(o_call, 30 if M <= 512 else 10), 2)
+        from kairos_amd.temp_cache import default_cache
+        shared = default_cache()
+        shared_bytes = int(getattr(shared, "capacity", 0) or 0)              # the one buffer every layer converts into
+        switched_bytes = sum(sum(getattr(layers[li][0], k).numel() * getattr(layers[li][0], k).element_size()
+                                 for k in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1"))
+                             for li in range(len(LAYER)))
+        oracle_bytes = sum(o_layers[li][0].resident_bytes() for li in range(len(LAYER)))
+        keep_all = {"oracle_keep_all_us_per_layer": round(o_us, 2),
+                    "switched_over_oracle": round(o_us / us_per_layer, 4),
+                    "meaning": "oracle time / switched time over the same 13-M step (the reference reports 0.93 on an A100)",
+                    "oracle_us_per_layer_by_m": o_by_m,
+                    "oracle_lane_by_shape_and_m": {f"{n}:{M}": lane for (n, M), lane in o_pick.items()},
+                    "hbm_bytes_per_layer_switched": switched_bytes,
+                    "hbm_bytes_shared_conversion_buffer": shared_bytes,
+                    "hbm_bytes_per_layer_oracle": oracle_bytes,
+                    "memory_switched_over_int4_only": round((switched_bytes * 32 + shared_bytes) / (switched_bytes * 32), 4),
+                    "memory_oracle_over_int4_only": round(oracle_bytes / switched_bytes, 4),
+                    "memory_note": "per layer: packed int4 + tables (switched) against int4 + tables + int8 + fp16 copies (oracle); the "
+                                   "switched model adds ONE shared conversion buffer for all its layers (ratio quoted for 32 layers)"}
+        del o_layers
+        torch.cuda.empty_cache()
 
     sweep = []
     if not args.no_sweep:
@@ -470,12 +565,13 @@ def main():
                    "converted_weight_cache": (f"LRU, {args.resident_cache_mb} MiB" if args.resident_cache_mb > 0
                                               else "one shared buffer (largest converted weight)"),
                    "lut_segments": prof.seg_perf_list},
-        "roofline": roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "roofline_all_kernels": roofline_all, "cpu_baseline": cpu,
         "wall_s_timed_region": round(wall, 3),
         "conversion_share_of_kernel_time": round(conv_sec / total_kernel_sec, 4),
         "replay_brackets_dropped_as_host_stalls": tracer.dropped,
         "kernels": kernels, "us_per_layer_by_m": by_m,
         "graph_replay_us_per_layer_by_m": graph_by_m,
+        "keep_all_oracle": keep_all,
         "best_small_m": small and {k: small[k] for k in ("shape", "M", "us", "gbps", "roofline_frac")},
         "best_large_m": large and {k: large[k] for k in ("shape", "M", "lane", "us", "tflops", "roofline_frac")},
         "config1_gemv_us": round(cfg1_us, 2),

@@ -16,7 +16,8 @@ class SwitchLinear(DynamicLinear):
 
     def init(self):
         super().init()
-        self._resident = None           # (int8 weight, fp16 weight, int8 row-major or None, tiled), built on first use
+        self._resident = None           # (int8 weight, fp16 weight, tiled), built on first use
+        self._w8_rows = None            # row-major int8 for the W8A16 lane, built when that lane is first asked for
 
     def _ensure_resident(self):
         """The int8 and fp16 copies are derived data: not part of state_dict, rebuilt after a load or a move."""
@@ -26,12 +27,14 @@ class SwitchLinear(DynamicLinear):
             ops.dequant_interleaved_int4_to_int8(w8, self.qweight, self.scales_to8, self.scaled_zeros_to8, 128, tiled=tiled)
             w16 = torch.empty(self.shape, dtype=torch.float16, device=dev)
             ops.dequant_interleaved_int4_to_fp16(w16, self.qweight, self.scales, self.scaled_zeros, 128, tiled=tiled)
-            w8_rows = None
-            if tiled:       # the W8A16 lane reads row-major int8
-                w8_rows = torch.empty(self.shape, dtype=torch.int8, device=dev)
-                ops.dequant_interleaved_int4_to_int8(w8_rows, self.qweight, self.scales_to8, self.scaled_zeros_to8, 128)
-            self._resident = (w8, w16, w8_rows, tiled)
+            self._resident = (w8, w16, tiled)
         return self._resident
+
+    def resident_bytes(self):
+        """Bytes of HBM this layer holds: the packed weight and its tables plus every converted copy built so far."""
+        held = [getattr(self, k) for k in ("qweight", "scales", "scaled_zeros", "scales_to8", "scaled_zeros_to8", "scales_1", "bias")]
+        held += list(getattr(self, "_resident", None) or ())[:2] + [getattr(self, "_w8_rows", None)]
+        return sum(t.numel() * t.element_size() for t in held if isinstance(t, torch.Tensor))
 
     @property
     def smq_weight(self):               # names of the reference's attributes (kairos/switch_linear.py:43-213)
@@ -50,7 +53,10 @@ class SwitchLinear(DynamicLinear):
         return q
 
     def _converted(self, fmt, tiled=None):
-        w8, w16, w8_rows, res_tiled = self._ensure_resident()
-        if fmt == 'i8' and tiled is False and res_tiled:
-            return w8_rows, False
+        w8, w16, res_tiled = self._ensure_resident()
+        if fmt == 'i8' and tiled is False and res_tiled:    # the W8A16 lane reads row-major int8
+            if getattr(self, "_w8_rows", None) is None:
+                self._w8_rows = torch.empty(self.shape, dtype=torch.int8, device=self.qweight.device)
+                ops.dequant_interleaved_int4_to_int8(self._w8_rows, self.qweight, self.scales_to8, self.scaled_zeros_to8, 128)
+            return self._w8_rows, False
         return (w8 if fmt == 'i8' else w16), res_tiled
