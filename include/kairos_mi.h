@@ -293,6 +293,24 @@ int kmi_lut_get(void* lut, int m);   /* comp_type, or KMI_E_HANDLE for a NULL/em
 int kmi_lut_shrink_to_fit(void* lut);
 int kmi_lut_size(void* lut);
 
+/* ---- bounded conversion buffer (host only) ------------------------------------------------------ */
+
+/* The lanes that convert on demand (W8A8, fp16, W8A16) write the converted weight into a temporary buffer; the
+ * reference allocates `torch.empty(self.shape)` per call and leaves the bound to the caching allocator
+ * (kairos/dynamic_linear.py:145,159).  A binder without such an allocator keeps ONE device buffer, sized for the largest
+ * converted weight of its model, and lets this handle do the bookkeeping: nothing here allocates or touches device
+ * memory.  kmi_cache_create wraps the caller's buffer (NULL on error).  kmi_cache_acquire(owner, format, nbytes): owner =
+ * any id unique to the layer, format = caller-defined (e.g. 1 int8 row-major, 2 int8 tiled, 3 fp16 row-major, 4 fp16
+ * tiled); returns 1 if the buffer already holds exactly that copy (skip the conversion), 0 if not (convert into
+ * *out_ptr now; the handle records the new content), KMI_E_SHAPE if nbytes exceeds the buffer -- the bound holds.
+ * kmi_cache_invalidate forgets the content (the buffer was used for something else, or the weights changed).  Use one
+ * handle per stream of execution; a hit is valid only for work ordered after the conversion that filled the buffer. */
+void* kmi_cache_create(void* device_buffer, size_t capacity_bytes);
+void kmi_cache_destroy(void* cache);
+int kmi_cache_acquire(void* cache, uint64_t owner, int format, size_t nbytes, void** out_ptr);
+int kmi_cache_invalidate(void* cache);
+int kmi_cache_stats(void* cache, size_t* capacity, size_t* high_water, uint64_t* hits, uint64_t* misses);
+
 #ifdef __cplusplus
 }
 #endif

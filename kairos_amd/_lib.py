@@ -58,8 +58,14 @@ SIGNATURES = {
     "kmi_lut_get": [_P, _I],
     "kmi_lut_shrink_to_fit": [_P],
     "kmi_lut_size": [_P],
+    "kmi_cache_create": [_P, _Z],
+    "kmi_cache_destroy": [_P],
+    "kmi_cache_acquire": [_P, ctypes.c_uint64, _I, _Z, ctypes.POINTER(_P)],
+    "kmi_cache_invalidate": [_P],
+    "kmi_cache_stats": [_P, ctypes.POINTER(_Z), ctypes.POINTER(_Z), ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)],
 }
 _RESTYPE = {"kmi_get_last_error_string": ctypes.c_char_p, "kmi_lut_new": _P, "kmi_lut_free": None,
+            "kmi_cache_create": _P, "kmi_cache_destroy": None,
             "kmi_gemm_force_tile": None, "kmi_gemm_force_splits": None}
 
 _lib = None

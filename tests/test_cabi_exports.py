@@ -180,3 +180,30 @@ def test_tile_queries_survive_empty_products(lib):
         assert lib.kmi_gemm_pick_tile(M, N, K) in (64, 128, 192, 256, 320)
         assert lib.kmi_gemm_w4a16_wp_rows(M, N, K) in (0, 32, 64, 128)
     assert lib.kmi_gemm_w4a8_pick_tile(16, 4096, 0) == 128
+
+
+def test_conversion_cache_handle_keeps_the_bound(lib):
+    """The C-side bookkeeping of the bounded conversion buffer: hits only for the very copy the buffer holds, a request
+    beyond the buffer is refused, invalidation forgets."""
+    import ctypes
+    assert not lib.kmi_cache_create(None, 1024) and not lib.kmi_cache_create(24, 1024) and not lib.kmi_cache_create(4096, 0)
+    c = lib.kmi_cache_create(4096, 1 << 20)
+    assert c
+    ptr = ctypes.c_void_p()
+    try:
+        assert lib.kmi_cache_acquire(c, 7, 2, 1 << 19, ctypes.byref(ptr)) == 0 and ptr.value == 4096      # miss: convert now
+        assert lib.kmi_cache_acquire(c, 7, 2, 1 << 19, ctypes.byref(ptr)) == 1                              # same copy: hit
+        assert lib.kmi_cache_acquire(c, 7, 3, 1 << 19, ctypes.byref(ptr)) == 0                              # other format
+        assert lib.kmi_cache_acquire(c, 8, 3, 1 << 19, ctypes.byref(ptr)) == 0                              # other layer
+        assert lib.kmi_cache_acquire(c, 8, 3, 1 << 19, ctypes.byref(ptr)) == 1
+        assert lib.kmi_cache_acquire(c, 8, 3, (1 << 20) + 16, ctypes.byref(ptr)) == -2                      # beyond the bound
+        assert b"asked of a buffer" in lib.kmi_get_last_error_string()
+        assert lib.kmi_cache_acquire(c, 8, 3, 1 << 19, ctypes.byref(ptr)) == 1                              # a refusal changes nothing
+        assert lib.kmi_cache_invalidate(c) == 0 and lib.kmi_cache_acquire(c, 8, 3, 1 << 19, ctypes.byref(ptr)) == 0
+        cap, high = ctypes.c_size_t(), ctypes.c_size_t()
+        hits, misses = ctypes.c_uint64(), ctypes.c_uint64()
+        assert lib.kmi_cache_stats(c, ctypes.byref(cap), ctypes.byref(high), ctypes.byref(hits), ctypes.byref(misses)) == 0
+        assert (cap.value, high.value, hits.value, misses.value) == (1 << 20, 1 << 19, 3, 4)
+        assert lib.kmi_cache_acquire(None, 1, 1, 16, ctypes.byref(ptr)) == -7 and lib.kmi_cache_acquire(c, 1, 1, 16, None) == -1
+    finally:
+        lib.kmi_cache_destroy(c)

@@ -436,6 +436,92 @@ def test_decoder_harness_two_layers(gpu):
         DynamicLinear.prof = old
 
 
+def test_decoder_harness_at_8b_width(gpu):
+    """The same harness at the true Llama-3-8B layer shapes (hidden 4096, 32 query / 8 key-value heads, MLP 14336), two
+    layers that share one set of prepared weights, batch 2, 64 prompt tokens + 4 decoded, with the committed MI355X
+    lookup table (so every linear runs the lane the benchmark runs at these token counts: the small-M kernel at M = 2,
+    the W4A16 GEMM and the W4A8 lane at M = 128).  Against the same stack on fp16 weights dequantised by the library's
+    converter, which is checked against the oracle on a slab of every weight; graph-replayed tokens equal eager ones."""
+    import os
+    from kairos.dynamic_linear_v2 import DynamicLinear
+    from kairos.perf_profiler_v2 import Profiler
+    from kairos_amd import ops
+    from kairos_amd.bench_extra import Decoder
+    dev = torch.device("cuda:0")
+    hidden, heads, kv, mlp, vocab = 4096, 32, 8, 14336, 4096
+    shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
+    prof = Profiler(shapes)
+    prof.load(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "kairos_amd", "prof", "llama3_8b_mi355x_v2") + "/")
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+
+    class Dense(torch.nn.Module):
+        def __init__(self, w16):
+            super().__init__()
+            self.w = w16
+
+        def forward(self, x):
+            return x @ self.w.T
+
+    try:
+        ql, dl_ = [], []
+        for i, (N, K) in enumerate(shapes):
+            w = torch.from_numpy(O.synth_weights(N, K, seed=200 + i) * np.float16(2.0)).cuda()
+            prepared = ops.prepare_weight(w)
+            q = DynamicLinear(K, N, False, dev, 128)
+            for key, val in prepared.items():
+                setattr(q, key, val)
+            ql.append(q)
+            w16 = torch.empty((N, K), dtype=torch.float16, device=dev)
+            ops.dequant_interleaved_int4_to_fp16(w16, q.qweight, q.scales, q.scaled_zeros, 128)
+            rows = slice(N // 2, N // 2 + 256)                                   # the converter against the oracle on a slab
+            want = O.dequant_to_f16(q.qweight[rows.start // 4:rows.stop // 4].cpu().numpy(), q.scales[:, rows].cpu().numpy(),
+                                    q.scaled_zeros[:, rows].cpu().numpy())
+            assert np.array_equal(w16[rows].cpu().numpy().view(np.uint16), want.view(np.uint16))
+            dl_.append(Dense(w16))
+        quant, dense = [ql, ql], [dl_, dl_]                                     # two layers, one set of prepared weights
+        B, prompt, t_max = 2, 64, 96
+        dec = Decoder(quant, dev, hidden, heads, kv, vocab, matched=True, t_max=t_max, seed=3)
+        ref = Decoder(dense, dev, hidden, heads, kv, vocab, matched=False, t_max=t_max, seed=3)
+
+        def rel(a, b):
+            return ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+
+        names = {v: k for k, v in __import__("kairos.dynamic_linear_v2", fromlist=["COMP_TYPE_NAME"]).COMP_TYPE_NAME.items()}
+        prefill_lanes = {names[prof.get_comp_type(s, B * prompt)] for s in shapes}
+        assert {names[prof.get_comp_type(s, B)] for s in shapes} == {"w4a16_gemv"}
+        ids = torch.randint(0, vocab, (B, prompt), device=dev, generator=torch.Generator(device=dev).manual_seed(5))
+        dec.alloc(B)
+        ref.alloc(B)
+        got, want = dec.prefill_logits(ids), ref.prefill_logits(ids)
+        # int8 activations (W4A8 / W8A8 lanes) in the prefill: a sanity bound; fp16-activation lanes only: the fp16 bar
+        tol = 0.15 if prefill_lanes & {"w4a8_qserve", "w8a8"} else 2e-2
+        assert torch.isfinite(got).all() and rel(got, want) < tol, (prefill_lanes, rel(got, want))
+        first = want.argmax(-1)
+        dec.start(first, prompt)
+        ref.start(first, prompt)
+        eager = []
+        for t in range(4):
+            dec.step()
+            ref.step()
+            # the decode steps (small-M lane) attend over the cache that the prefill's lanes wrote: the prefill's bound
+            assert rel(dec.logits, ref.logits) < tol, (t, rel(dec.logits, ref.logits))
+            eager.append((dec.tok.clone(), dec.logits.clone()))
+            ref.x_in.copy_(dec.x_in)                # keep the two sequences on the same tokens
+        graph = dec.capture()
+        dec.prefill_logits(ids)
+        dec.start(first, prompt)
+        for t in range(4):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(dec.tok, eager[t][0]), f"token {t}: graph replay and eager decoding disagree"
+            assert torch.equal(dec.logits.view(torch.int16), eager[t][1].view(torch.int16))
+        dec.free()
+        ref.free()
+    finally:
+        DynamicLinear.prof = old
+
+
 def test_smooth_scale_search_with_the_library_probe(gpu):
     """The smoothing-scale search (kairos/smooth_scale.py:66-176) with its default probe -- the library's own quantised
     linear through the W4A8 lane -- on a tiny fp16 Llama with outlier channels: the scales it finds lower the error of
