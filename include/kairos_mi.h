@@ -293,6 +293,17 @@ int kmi_lut_get(void* lut, int m);   /* comp_type, or KMI_E_HANDLE for a NULL/em
 int kmi_lut_shrink_to_fit(void* lut);
 int kmi_lut_size(void* lut);
 
+/* ---- measurement probes ------------------------------------------------------------------------- */
+
+/* Kernels that only read, for the floors the streaming kernels are measured against; no product path calls them and
+ * nothing in the reference corresponds to them.  kmi_probe_empty: one empty launch of 256 workgroups.
+ * kmi_probe_stream_read: a plain reader of `bytes` bytes, 16 contiguous KiB per workgroup.  kmi_probe_gemv_read: exactly
+ * the weight loads of kmi_gemv_w4a16's register form with nt column tiles per wave and nw waves per workgroup
+ * (kmi_gemv_w4a16_plan reports what a call uses), no activations, tables, arithmetic or stores. */
+int kmi_probe_empty(void* stream);
+int kmi_probe_stream_read(const void* buf, size_t bytes, void* stream);
+int kmi_probe_gemv_read(const void* qweight, int N, int K, int nt, int nw, void* stream);
+
 /* ---- bounded conversion buffer (host only) ------------------------------------------------------ */
 
 /* The lanes that convert on demand (W8A8, fp16, W8A16) write the converted weight into a temporary buffer; the

@@ -58,6 +58,9 @@ SIGNATURES = {
     "kmi_lut_get": [_P, _I],
     "kmi_lut_shrink_to_fit": [_P],
     "kmi_lut_size": [_P],
+    "kmi_probe_empty": [_P],
+    "kmi_probe_stream_read": [_P, _Z, _P],
+    "kmi_probe_gemv_read": [_P, _I, _I, _I, _I, _P],
     "kmi_cache_create": [_P, _Z],
     "kmi_cache_destroy": [_P],
     "kmi_cache_acquire": [_P, ctypes.c_uint64, _I, _Z, ctypes.POINTER(_P)],

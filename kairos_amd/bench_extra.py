@@ -98,6 +98,74 @@ def gemv70b(args):
             "whole_model_int4_gb": round(whole_model_gb, 1)}
 
 
+def _graph_time(fn, n=40, reps=3):
+    """us per launch of `fn(i, raw_stream)` with n launches recorded into one HIP graph: back-to-back device time, no
+    host launch cost between the kernels."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(3):
+            fn(i, side.cuda_stream)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        for i in range(n):
+            fn(i, side.cuda_stream)
+    best = float("inf")
+    for _ in range(reps):
+        g.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) * 1e3 / n)
+    return best
+
+
+def floor(args):
+    """What a streaming launch costs at the sizes of the small-M lane, beside the small-M kernel itself: an empty
+    launch, a plain reader of the weight's bytes, a reader that issues the kernel's own weight loads and nothing else,
+    and the kernel at M = 1, 4, 8, 16, 32.  All graph-replayed (device time between back-to-back launches), weights
+    rotated through more than 700 MB so that none is found in the last-level cache."""
+    from . import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    out = {"bench": "floor", "unit": "us per launch (HIP-graph replay of 40 back-to-back launches, best of 3)",
+           "empty_launch_us": round(_graph_time(lambda i, st: lib.kmi_probe_empty(st)), 2), "rows": []}
+    shapes = [("8b_qkv", 6144, 4096), ("8b_o", 4096, 4096), ("8b_gate_up", 28672, 4096), ("8b_down", 4096, 14336),
+              ("70b_qkv", 10240, 8192), ("70b_gate_up", 57344, 8192), ("70b_down", 8192, 28672)]
+    ws = ops.gemv_workspace_for(dev)
+    for name, N, K in shapes:
+        copies = max(2, math.ceil(700e6 / (N * K / 2)))
+        gp = ((K // 128 + 7) // 8) * 8
+        qw = [torch.randint(-32768, 32767, (N // 4, K), dtype=torch.int16, device=dev) for _ in range(copies)]
+        sc = torch.rand((gp, N), dtype=torch.float16, device=dev) * 0.01
+        sz = torch.rand((gp, N), dtype=torch.float16, device=dev) * -0.08
+        nbytes = N * K // 2
+        row = {"shape": name, "N": N, "K": K, "weight_mb": round(nbytes / 1e6, 1),
+               "plain_reader_us": round(_graph_time(lambda i, st: lib.kmi_probe_stream_read(qw[i % copies].data_ptr(), nbytes, st)), 2)}
+        for M in (1, 4, 8, 16, 32):
+            plan = ops.gemv_plan(M, N, K)
+            x = torch.randn((M, K), dtype=torch.float16, device=dev)
+            y = torch.empty((M, N), dtype=torch.float16, device=dev)
+            us = _graph_time(lambda i, st: _lib.check(lib.kmi_gemv_w4a16(y.data_ptr(), x.data_ptr(), qw[i % copies].data_ptr(), sc.data_ptr(),
+                                                                        sz.data_ptr(), None, M, N, K, 128, ws.data_ptr(), ws.numel(), st)))
+            b = nbytes + 4 * (K // G) * N + 2 * M * K + 2 * M * N
+            row[f"M{M}"] = {"us": round(us, 2), "hbm_frac": round(b / us / 1e-6 / HBM, 3), "form": plan["form"],
+                            "nt": plan["nt"], "nw": plan["nw"], "ks": plan["ks"]}
+            if M == 1:        # the kernel's own weight loads, nothing else (the register form's lanes; unsplit)
+                nw = plan["nw"] if plan["nw"] in (4, 8, 16) else 8
+                row["own_loads_reader_us"] = round(_graph_time(
+                    lambda i, st: lib.kmi_probe_gemv_read(qw[i % copies].data_ptr(), N, K, plan["nt"], nw, st)), 2)
+        out["rows"].append(row)
+        print(row, file=sys.stderr, flush=True)
+        del qw
+        torch.cuda.empty_cache()
+    return out
+
+
 def convert(args):
     """On-demand conversion on Qwen2.5-7B shapes; int4 -> int8, fp16, tiled; temp-cache high-water mark."""
     dev = torch.device("cuda:0")
@@ -563,6 +631,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
     sub.add_parser("gemv70b")
+    sub.add_parser("floor")
     sub.add_parser("convert")
     sub.add_parser("weightprep")
     sub.add_parser("blasref")
@@ -583,7 +652,7 @@ def main(argv=None):
     if args.cmd == "decoder" and args.lut is None:
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x_v2") + "/"
-    res = {"gemv70b": gemv70b, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "floor": floor, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libkairos_mi.so")
-SOURCES = ["api.cpp", "cvt_i4.hip", "quant_act.hip", "norm_quant.hip", "prep_w8a8.hip", "weight_prep.hip", "trans_layout.hip", "gemv_w4a16.hip", "gemm_mfma.hip", "gemm_w4a8.hip"]
+SOURCES = ["api.cpp", "cvt_i4.hip", "quant_act.hip", "norm_quant.hip", "prep_w8a8.hip", "weight_prep.hip", "trans_layout.hip", "gemv_w4a16.hip", "gemm_mfma.hip", "gemm_w4a8.hip", "probes.hip"]
 HEADERS = [os.path.join(CSRC, "kmi_common.h"), os.path.join(CSRC, "prep_bodies.h"), os.path.join(CSRC, "gemm_parts.h"), os.path.join(os.path.dirname(HERE), "include", "kairos_mi.h")]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-unused-command-line-argument",
          "-Wno-pass-failed", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-x", "hip"]

@@ -33,33 +33,44 @@
 #include <mutex>
 #include <set>
 
-// Tail shared by the kernels of this file: the waves' partial tiles meet in LDS (`red`, nw * MT*NT*4 * 64 floats)
+// Row spread.  With at most four activation rows the kernels place row m in row 4m of the 16-row MFMA operand
+// (RS = 4; RS = 2 for up to eight rows), so that the rows that count land in accumulator element 0 (elements 0 and 2)
+// of the lanes: the per-group scale-and-add then touches one (two) of the four accumulator registers of a tile, and
+// the reduction moves a quarter (half) of the data.  RS = 1 is the plain layout.
+//
+// Tail shared by the kernels of this file: the waves' partial tiles meet in LDS (`red`, nw * MT*NT*(4/RS) * 64 floats)
 // and are added in wave order; with a split over K (gridDim.y > 1) the workgroup's sums go to `partial`, the
 // strip's arrival counter is bumped and whichever workgroup arrives last adds the slices in split order.
-template <int MT, int NT>
+template <int MT, int NT, int RS>
 __device__ __forceinline__ void gemv_finish(const f4_t (&acc)[MT][NT], float* red, int NW, int wave, int lane, int strip, int n0,
                                             half_t* __restrict__ out, const half_t* __restrict__ bias, int M, int N,
                                             float* __restrict__ partial, uint32_t* __restrict__ counters) {
     const int KS = gridDim.y, ks = blockIdx.y;
-    constexpr int R = MT * NT * 4;
+    constexpr int E = 4 / RS;                                // live accumulator elements per tile
+    constexpr int R = MT * NT * E;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[(wave * R + (mt * NT + nt) * 4 + i) * 64 + lane] = acc[mt][nt][i];
+            for (int e = 0; e < E; ++e) red[(wave * R + (mt * NT + nt) * E + e) * 64 + lane] = acc[mt][nt][e * RS];
     __syncthreads();
+    // idx -> (lane l, live element e of tile (mt, nt)); MFMA row 4*(l>>4) + e*RS holds activation row (that row) / RS
+    auto place = [&](int idx, int& m, int& n) {
+        const int l = idx & 63, reg = idx >> 6;
+        const int e = reg % E, t = reg / E;
+        const int nt = t % NT, mt = t / NT;
+        m = mt * 16 + (4 * (l >> 4) + e * RS) / RS;
+        n = n0 + nt * 16 + (l & 15);
+    };
 
     if (KS == 1) {
         for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
             float v = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
-            const int l = idx & 63, reg = idx >> 6;
-            const int i = reg & 3, t = reg >> 2;
-            const int nt = t % NT, mt = t / NT;
-            const int m = mt * 16 + 4 * (l >> 4) + i;
-            const int n = n0 + nt * 16 + (l & 15);
+            int m, n;
+            place(idx, m, n);
             if (m < M && n < N) {
                 half_t h = (half_t)v;
                 if (bias) h = (half_t)((float)h + (float)bias[n]);
@@ -73,14 +84,16 @@ __device__ __forceinline__ void gemv_finish(const f4_t (&acc)[MT][NT], float* re
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) v += red[w * R * 64 + idx];
-        const int l = idx & 63, reg = idx >> 6;
-        const int i = reg & 3, t = reg >> 2;
-        const int nt = t % NT, mt = t / NT;
-        const int m = mt * 16 + 4 * (l >> 4) + i;
-        const int n = n0 + nt * 16 + (l & 15);
+        int m, n;
+        place(idx, m, n);
         if (m < M && n < N)
             __hip_atomic_store(partial + ((long)ks * M + m) * N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    // Hand-off without fences.  Every partial sum travels by an agent-scope atomic store (performed at the memory side
+    // that all XCDs share, not in this XCD's L2); `s_waitcnt vmcnt(0)` holds the thread until its stores have been
+    // performed, the barrier until every thread's have; only then is the arrival counted, by an agent-scope atomic add
+    // at the same memory side.  A workgroup that reads KS-1 from the counter therefore runs after every other
+    // workgroup's stores were performed, and its agent-scope atomic loads read them from that memory side.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this thread's partial sums have been performed
     __shared__ uint32_t arrived;
     __syncthreads();                                         // ... and everybody else's in the workgroup
@@ -88,11 +101,8 @@ __device__ __forceinline__ void gemv_finish(const f4_t (&acc)[MT][NT], float* re
     __syncthreads();
     if (arrived != (uint32_t)(KS - 1)) return;               // workgroup-uniform
     for (int idx = threadIdx.x; idx < R * 64; idx += NW * 64) {
-        const int l = idx & 63, reg = idx >> 6;
-        const int i = reg & 3, t = reg >> 2;
-        const int nt = t % NT, mt = t / NT;
-        const int m = mt * 16 + 4 * (l >> 4) + i;
-        const int n = n0 + nt * 16 + (l & 15);
+        int m, n;
+        place(idx, m, n);
         if (m < M && n < N) {
             float v = 0.f;
             for (int q = 0; q < KS; ++q)                     // split order: the same sum whoever arrives last
@@ -105,14 +115,15 @@ __device__ __forceinline__ void gemv_finish(const f4_t (&acc)[MT][NT], float* re
     if (threadIdx.x == 0) __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
-template <int MT, int NT, int NW>
+template <int MT, int NT, int NW, int RS>
 __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict__ out, const half_t* __restrict__ x,
                                                              const u4_t* __restrict__ qw,
                                                              const half_t* __restrict__ scales,
                                                              const half_t* __restrict__ szeros,
                                                              const half_t* __restrict__ bias, int M, int N, int K,
                                                              float* __restrict__ partial, uint32_t* __restrict__ counters) {
-    extern __shared__ float red[];               // [NW][MT*NT*4][64]
+    static_assert(RS == 1 || MT == 1, "rows are spread over the operand only when one row tile holds them all");
+    extern __shared__ float red[];               // [NW][MT*NT*(4/RS)][64]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int r16 = lane & 15;
@@ -151,8 +162,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
     bool xrow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + r16;
-        xrow[mt] = m < M;
+        const int m = mt * 16 + r16 / RS;                    // operand row r16 carries activation row r16 / RS ...
+        xrow[mt] = m < M && (r16 % RS) == 0;                 // ... if it is a multiple of the spread
         xp[mt] = reinterpret_cast<const h8_t*>(x) + (long)(xrow[mt] ? m : 0) * kq + j * 4;
     }
 
@@ -223,7 +234,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
                         pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][2], __builtin_bit_cast(h8_t, lo8), pg, 0, 0, 0);
                         pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][mt][3], __builtin_bit_cast(h8_t, hi8), pg, 0, 0, 0);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
+                        for (int i = 0; i < 4; i += RS)          // the rows that count (see the row spread above)
                             acc[mt][nt][i] = __builtin_fmaf(pg[i], sc, __builtin_fmaf(xsum[mt][i], zc, acc[mt][nt][i]));
                     }
                 }
@@ -231,7 +242,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_w4a16_kernel(half_t* __restrict_
         }
     }
 
-    gemv_finish<MT, NT>(acc, red, NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
+    gemv_finish<MT, NT, RS>(acc, red, NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
 }
 
 // =====================================================================================================================
@@ -272,6 +283,7 @@ __global__ __launch_bounds__(512) void gemv_ring_kernel(half_t* __restrict__ out
                                                         uint32_t* __restrict__ counters) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass cannot instantiate code that uses the buffer resource type
     constexpr int MT = (XI + 3) / 4;
+    constexpr int RS = XI == 1 ? 4 : XI == 2 ? 2 : 1;              // row spread: at most 4 / 8 rows sit in operand rows 4m / 2m
     constexpr int L = NT + XI + 2;                                 // direct loads per slot
     constexpr int X_OFF = NT * 1024, S_OFF = X_OFF + XI * 1024, SLOT = S_OFF + 512;
     constexpr int KMAX = gemv_ring_max_depth<XI, NT>() - 1;
@@ -331,7 +343,7 @@ __global__ __launch_bounds__(512) void gemv_ring_kernel(half_t* __restrict__ out
     int xoff[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        int row = mt * 16 + r16;
+        int row = mt * 16 + r16 / RS;                              // operand row r16 carries activation row r16 / RS
         row = row < 4 * XI ? row : 4 * XI - 1;
 #pragma unroll
         for (int a = 0; a < 4; ++a) xoff[mt][a] = X_OFF + (row * 16 + ((4 * j + a) ^ (row & 15))) * 16;
@@ -400,7 +412,7 @@ __global__ __launch_bounds__(512) void gemv_ring_kernel(half_t* __restrict__ out
                 pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][2], __builtin_bit_cast(h8_t, lo8), pg, 0, 0, 0);
                 pg = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][3], __builtin_bit_cast(h8_t, hi8), pg, 0, 0, 0);
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
+                for (int e = 0; e < 4; e += RS)                     // the rows that count
                     acc[mt][nt][e] = __builtin_fmaf(pg[e], sc, __builtin_fmaf(xsum[mt][e], zc, acc[mt][nt][e]));
             }
         }
@@ -408,7 +420,7 @@ __global__ __launch_bounds__(512) void gemv_ring_kernel(half_t* __restrict__ out
     // every wave has emptied its ring (and no direct load is outstanding) before the rings become the reduction buffer
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    gemv_finish<MT, NT>(acc, reinterpret_cast<float*>(smem), NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
+    gemv_finish<MT, NT, RS>(acc, reinterpret_cast<float*>(smem), NW, wave, lane, strip, n0, out, bias, M, N, partial, counters);
 #endif
 }
 
@@ -419,43 +431,53 @@ static constexpr bool gemv_cfg_ok() {
     return MT * NT <= 8 && NW * MT * NT <= 64 && (NW < 16 || MT * NT <= 2);
 }
 
+static int gemv_row_spread(int M) { return M <= 4 ? 4 : M <= 8 ? 2 : 1; }
+
 template <int MT, int NT, int NW>
-static gemv_fn gemv_pick() {
-    if constexpr (gemv_cfg_ok<MT, NT, NW>()) return gemv_w4a16_kernel<MT, NT, NW>;
-    else return nullptr;
+static gemv_fn gemv_pick(int rs) {
+    if constexpr (gemv_cfg_ok<MT, NT, NW>()) {
+        if constexpr (MT == 1) {
+            if (rs == 4) return gemv_w4a16_kernel<MT, NT, NW, 4>;
+            if (rs == 2) return gemv_w4a16_kernel<MT, NT, NW, 2>;
+        }
+        return gemv_w4a16_kernel<MT, NT, NW, 1>;
+    } else {
+        return nullptr;
+    }
 }
 
 template <int MT, int NT>
-static gemv_fn gemv_pick_nw(int nw) {
+static gemv_fn gemv_pick_nw(int nw, int rs) {
     switch (nw) {
-        case 4: return gemv_pick<MT, NT, 4>();
-        case 8: return gemv_pick<MT, NT, 8>();
-        case 16: return gemv_pick<MT, NT, 16>();
+        case 4: return gemv_pick<MT, NT, 4>(rs);
+        case 8: return gemv_pick<MT, NT, 8>(rs);
+        case 16: return gemv_pick<MT, NT, 16>(rs);
     }
     return nullptr;
 }
 
 template <int MT>
-static gemv_fn gemv_pick_nt(int nt, int nw) {
+static gemv_fn gemv_pick_nt(int nt, int nw, int rs) {
     switch (nt) {
-        case 1: return gemv_pick_nw<MT, 1>(nw);
-        case 2: return gemv_pick_nw<MT, 2>(nw);
-        case 3: return gemv_pick_nw<MT, 3>(nw);
-        case 4: return gemv_pick_nw<MT, 4>(nw);
-        case 5: return gemv_pick_nw<MT, 5>(nw);
-        case 6: return gemv_pick_nw<MT, 6>(nw);
-        case 7: return gemv_pick_nw<MT, 7>(nw);
-        case 8: return gemv_pick_nw<MT, 8>(nw);
+        case 1: return gemv_pick_nw<MT, 1>(nw, rs);
+        case 2: return gemv_pick_nw<MT, 2>(nw, rs);
+        case 3: return gemv_pick_nw<MT, 3>(nw, rs);
+        case 4: return gemv_pick_nw<MT, 4>(nw, rs);
+        case 5: return gemv_pick_nw<MT, 5>(nw, rs);
+        case 6: return gemv_pick_nw<MT, 6>(nw, rs);
+        case 7: return gemv_pick_nw<MT, 7>(nw, rs);
+        case 8: return gemv_pick_nw<MT, 8>(nw, rs);
     }
     return nullptr;
 }
 
-static gemv_fn gemv_lookup(int mt, int nt, int nw) {
+// rs: row spread of the kernel (gemv_row_spread(M)); the existence of a kernel does not depend on it
+static gemv_fn gemv_lookup(int mt, int nt, int nw, int rs = 1) {
     switch (mt) {
-        case 1: return gemv_pick_nt<1>(nt, nw);
-        case 2: return gemv_pick_nt<2>(nt, nw);
-        case 3: return gemv_pick_nt<3>(nt, nw);
-        case 4: return gemv_pick_nt<4>(nt, nw);
+        case 1: return gemv_pick_nt<1>(nt, nw, rs);
+        case 2: return gemv_pick_nt<2>(nt, nw, 1);
+        case 3: return gemv_pick_nt<3>(nt, nw, 1);
+        case 4: return gemv_pick_nt<4>(nt, nw, 1);
     }
     return nullptr;
 }
@@ -720,7 +742,8 @@ extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* 
                                     workspace_bytes, stream);
     }
     if (ks < 1) ks = 1;
-    gemv_fn fn = gemv_lookup(mt, nt, nw);
+    const int rs = mt == 1 ? gemv_row_spread(M) : 1;
+    gemv_fn fn = gemv_lookup(mt, nt, nw, rs);
     if (!fn) return kmi_set_error(KMI_E_SHAPE, "kmi_gemv_w4a16: no kernel for m-tiles=%d nt=%d nw=%d", mt, nt, nw);
     const int strips = N / 16, wg_x = (strips + nt - 1) / nt, groups = K / 128;
     // a split over K needs scratch: [KMI_GEMV_WS_HEADER bytes of per-strip arrival counters, zero between calls]
@@ -732,7 +755,7 @@ extern "C" int kmi_gemv_w4a16_cfg(void* out_f16, const void* x_f16, const void* 
         ks = 1;
     }
     const dim3 grid(wg_x, ks), block(nw * 64);
-    const size_t lds = (size_t)nw * mt * nt * 4 * 64 * sizeof(float);
+    const size_t lds = (size_t)nw * mt * nt * (4 / rs) * 64 * sizeof(float);
     uint32_t* counters = static_cast<uint32_t*>(workspace);
     float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + KMI_GEMV_WS_HEADER) : nullptr;
     hipLaunchKernelGGL(fn, grid, block, lds, static_cast<hipStream_t>(stream), static_cast<half_t*>(out_f16),

@@ -240,6 +240,25 @@ def quantize_int4_kairos(w8, group_size=GROUP):
         return q.reshape(shape).astype(np.int8), scale.astype(np.float16), zero.astype(np.float16)
 
 
+def quantize_int4_int_factors(w8, group_size=GROUP):
+    """The integer second-level factors that the version-2 quantiser also returns (kairos/dynamic_linear_v2.py:36-41):
+    scale_i = floor(scale_f), zero_pt_i = round_half_even(zero_pt_f), both taken from the fp32 values (before their
+    fp16 rounding) and stored as int8.  The reference computes them and nothing in its tree reads them; they describe
+    the W4A8 operand a per-group integer dequantiser would use.  Groups whose zero-point leaves the int8 range (constant
+    groups: scale 1e-5 / 15) have no defined int8 value there (the cast of an out-of-range float); they are returned
+    saturated and flagged in the third result.  -> (scale_i int8 [G,1], zero_pt_i int8 [G,1], in_range bool [G,1])"""
+    w8 = np.asarray(w8)
+    assert w8.shape[-1] % group_size == 0
+    x = w8.reshape(-1, group_size).astype(np.float32)
+    mx = x.max(axis=1, keepdims=True)
+    mn = x.min(axis=1, keepdims=True)
+    scale = np.maximum(mx - mn, np.float32(1e-5)) / np.float32(15)
+    zero = -(mn / scale)
+    zi = np.rint(zero)
+    in_range = (zi >= -128) & (zi <= 127)
+    return np.floor(scale).astype(np.int8), np.clip(zi, -128, 127).astype(np.int8), in_range
+
+
 def prepare_weights(w, group_size=GROUP):
     """kairos/dynamic_linear.py:86-115 (from_module): fp16 [N, K] -> dict of resident tensors."""
     w = np.asarray(w, dtype=np.float16)

@@ -49,3 +49,31 @@ def test_int8_and_int4_steps():
     assert cfg4["zero_pt_i"].dtype == torch.int8 and cfg4["scale_i"].dtype == torch.int8
     with pytest.raises(ValueError):
         W.kairos_quantize_tensor_int4(q8[:, :100], group_size=128)
+
+
+def test_integer_second_level_factors():
+    """scale_i = floor(scale_f), zero_pt_i = round(zero_pt_f) of the version-2 quantiser (kairos/dynamic_linear_v2.py:36-41):
+    the host mirror against the oracle, and the oracle against hand cases -- a group spanning -120..105 has scale 15 and
+    zero-point 8 exactly; -128..127 gives scale floor(17) and zero round(7.529) = 8; a half-way zero-point rounds to even."""
+    import numpy as np
+    import torch
+    from oracle import kairos_oracle as O
+    from kairos_amd import weight_prep as W
+    hand = np.zeros((3, 128), dtype=np.int8)
+    hand[0, :2] = (-120, 105)              # range 225: scale 15, zero 120 / 15 = 8
+    hand[1, :2] = (-128, 127)              # range 255: scale 17, zero 128 / 17 = 7.53
+    hand[2, :2] = (-75, 75)                # range 150: scale 10, zero 7.5 -> 8 (half to even)
+    si, zi, ok = O.quantize_int4_int_factors(hand)
+    assert si.reshape(-1).tolist() == [15, 17, 10] and zi.reshape(-1).tolist() == [8, 8, 8] and ok.all()
+    hand[2, :2] = (-65, 85)                # scale 10, zero 6.5 -> 6
+    assert O.quantize_int4_int_factors(hand)[1].reshape(-1).tolist() == [8, 8, 6]
+    w8 = np.random.default_rng(3).integers(-128, 128, size=(16, 512), dtype=np.int8)
+    w8[5, 128:256] = 33                    # a constant group: its zero-point leaves the int8 range
+    si, zi, ok = O.quantize_int4_int_factors(w8)
+    _q, cfg = W.kairos_quantize_tensor_int4(torch.from_numpy(w8), group_size=128)
+    assert np.array_equal(cfg["scale_i"].numpy(), si)
+    assert not ok[5 * 4 + 1] and ok.sum() == ok.size - 1
+    assert np.array_equal(cfg["zero_pt_i"].numpy()[ok], zi[ok])          # where the int8 value is defined
+    # consistency with the float factors the lanes use: |scale_f - scale_i| < 1, |zero_pt_f - zero_pt_i| <= 0.5 (+ fp16 rounding)
+    assert np.all(cfg["scale_f"].numpy().astype(np.float32)[ok] - si[ok] < 1.01)
+    assert np.all(np.abs(cfg["zero_pt_f"].numpy().astype(np.float32)[ok] - zi[ok]) <= 0.51)
