@@ -583,11 +583,12 @@ static GemvRingKernel gemv_ring_lookup(int M, int nt) {
 //   23.2, 4096 x 14336 18.5 -> 16.6, 10240 x 8192 20.5 -> 17.2, 57344 x 8192 80 -> 72, 8192 x 28672 41.7 -> 38.4,
 //   3584 x 18944 31.1 -> 19.4.  Column tiles per wave: one per 256 strips (so that about one workgroup lands on each
 //   CU), as many as the accumulators allow beyond.
-//   M <= 16 on narrow weights (at most 320 column strips) from M = 8, or from M = 1 where K is long (>= 96 groups):
-//   4096 x 4096 M=8 5.8 -> 5.5, M=16 6.7 -> 6.2; 4608 x 3584 M=16 7.2 -> 6.6; 4096 x 14336 M=1 9.9 -> 9.5, M=16 12.8 ->
-//   12.2; 3584 x 18944 M=16 19.4 -> 14.3.  Wide weights (28672, 37888, 57344 columns) stay with the register form there
-//   (12.8 against 14.6 us at 28672 x 4096): their trips are long enough to cover the wait, and the ring's extra hop
-//   through LDS costs more than it hides.
+//   M <= 16 on narrow weights: from M = 9 up to 640 column strips (6144 x 4096 M=16 7.3 -> 6.1, 10240 x 8192 13.7 ->
+//   13.3), from M = 5 up to 384 (4096 x 4096 M=8 5.4 -> 4.9, M=16 6.9 -> 5.5; 4608 x 3584 M=8 5.8 -> 5.2, M=16 7.4 -> 5.7),
+//   from M = 1 up to 320 where K is long (>= 96 groups: 4096 x 14336 M=1 9.9 -> 9.4, M=16 13.2 -> 12.4; 3584 x 18944
+//   M=16 15.0 -> 14.2).  Wide weights (28672, 37888, 57344 columns) stay with the register form there (12.2 against
+//   13.6 us at 28672 x 4096), as do long, fairly wide ones (8192 x 28672 up to M = 16: 22.5 against 24.9 us at M = 4):
+//   their trips are long enough to cover the wait, and the ring's extra hop through LDS costs more than it hides.
 //   Long K (>= 96 groups) at M >= 8: two workgroups share a strip's K range and the waves take twice the column tiles,
 //   which halves the activation bytes every CU pulls through its L1.
 static bool gemv_ring_default(int M, int N, int K, bool can_split, int* nt, int* nw, int* ks, int* depth) {
@@ -606,8 +607,10 @@ static bool gemv_ring_default(int M, int N, int K, bool can_split, int* nt, int*
         }
         return true;
     }
-    if (strips > 320 || !(M >= 8 || groups >= 96)) return false;
-    if (M >= 8 && long_k) {
+    // up to 16 rows: narrow weights only, and the narrower the fewer rows it takes for the ring to win
+    const int widest = M >= 9 ? ((groups >= 96) ? 320 : 640) : M >= 5 ? 384 : 320;
+    if (strips > widest || !(M >= 5 || groups >= 96)) return false;
+    if (M >= 8 && long_k && strips <= 320) {
         *nt = 2;
         *ks = 2;
     }

@@ -236,6 +236,11 @@ def main(argv=None):
     ap.add_argument("--preheat", type=int, default=20)
     ap.add_argument("--max-m", type=int, default=30720)
     ap.add_argument("--v2", action="store_true", help="version-2 id table and candidates (adds the W4A8 lane, id 7)")
+    ap.add_argument("--rotate-mb", type=int, default=512,
+                    help="rotate over layer copies whose packed weights add up to this many MiB (0 = time one layer over and over, as the reference does)")
+    ap.add_argument("--head-start-ms", type=float, default=4.0,
+                    help="queue the timed calls behind an idle kernel of this length so that device time is measured (0 = as the reference does)")
+    ap.add_argument("--stickiness", type=float, default=0.01, help="keep the previous M's lane within this fraction of the choice (0 = strict minimum)")
     ap.add_argument("--prefer-resident", type=float, default=0.0,
                     help="take a lane that reads only the int4 weight while it is within this fraction of the fastest (0 = strict minimum)")
     args = ap.parse_args(argv)
@@ -247,7 +252,8 @@ def main(argv=None):
         ProfilerCls = Profiler
     prof = ProfilerCls(PRESETS[args.preset])
     details = []
-    prof.profiling(input_len=grid, n=args.n, preheat_time=args.preheat, details=details, prefer_resident=args.prefer_resident)
+    prof.profiling(input_len=grid, n=args.n, preheat_time=args.preheat, details=details, prefer_resident=args.prefer_resident,
+                   rotate_bytes=args.rotate_mb << 20, head_start_ms=args.head_start_ms, stickiness=args.stickiness)
     out = args.out if args.out.endswith("/") else args.out + "/"
     prof.save(out)
     save_json(os.path.join(out, "timings.json"), details)

@@ -159,7 +159,10 @@ def test_small_m_plan_is_host_logic(lib):
     assert plan(1, 28672, 4096)["form"] == "register" and plan(16, 28672, 4096)["form"] == "register"
     assert plan(32, 28672, 4096) == {"form": "ring", "nt": 4, "nw": 8, "ks": 1, "depth": 2}
     assert plan(1, 4096, 4096)["form"] == "register" and plan(8, 4096, 4096)["form"] == "ring"
-    assert plan(16, 6144, 4096)["form"] == "register" and plan(32, 6144, 4096)["nt"] == 2
+    assert plan(4, 6144, 4096)["form"] == "register" and plan(8, 6144, 4096)["form"] == "ring"
+    assert plan(16, 6144, 4096) == {"form": "ring", "nt": 2, "nw": 8, "ks": 1, "depth": 2} and plan(32, 6144, 4096)["nt"] == 2
+    assert plan(16, 10240, 8192)["form"] == "ring" and plan(8, 10240, 8192)["form"] == "register"
+    assert plan(16, 8192, 28672)["form"] == "register" and plan(32, 8192, 28672)["form"] == "ring"
     assert plan(1, 4096, 14336) == {"form": "ring", "nt": 1, "nw": 8, "ks": 1, "depth": 2}
     assert plan(16, 4096, 14336) == {"form": "ring", "nt": 2, "nw": 8, "ks": 2, "depth": 2}
     assert plan(16, 4096, 14336, 0)["ks"] == 1 and plan(16, 4096, 14336, 0)["form"] == "ring"      # no scratch, no split

@@ -349,6 +349,31 @@ def test_split_k_result_does_not_depend_on_the_calling_thread(gpu):
     assert torch.equal(other.view(torch.int16), main.view(torch.int16))
 
 
+def test_forward_rejects_a_wrong_input_width(gpu):
+    """The decode fast path hands raw pointers to the library: an input whose last dimension is not the layer's K must
+    be refused on the host, in both the fast path and the general one, before any kernel reads past the buffer."""
+    from kairos.dynamic_linear import DynamicLinear
+    from kairos.perf_profiler import Profiler
+    N, K = 256, 512
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16)
+    dl = DynamicLinear.from_module(lin.cuda(), "cuda")
+    prof = Profiler([(N, K)])
+    prof.record_best_comp((N, K), 64, "w4a16_gemv")
+    prof.record_best_comp((N, K), 1 << 20, "w4a16_gemm")
+    old = DynamicLinear.prof
+    DynamicLinear.prof = prof
+    try:
+        assert dl(torch.zeros((1, 4, K), dtype=torch.float16, device="cuda")).shape == (1, 4, N)
+        with pytest.raises(ValueError):
+            dl(torch.zeros((1, 4, K // 2), dtype=torch.float16, device="cuda"))           # small-M fast path
+        from kairos_amd import ops
+        with pytest.raises(ValueError):
+            ops.gemv_forward(torch.zeros((4, K // 2), dtype=torch.float16, device="cuda"), dl.qweight, dl.scales,
+                             dl.scaled_zeros, 4, N, K)
+    finally:
+        DynamicLinear.prof = old
+
+
 def test_decoder_harness_two_layers(gpu):
     """The end-to-end decoder harness (GQA attention over a static KV cache, matched norm and SiLU operators, every
     linear a LUT-switched DynamicLinear, decode step replayed from a HIP graph) at reduced width, two layers:

@@ -463,3 +463,50 @@ def test_matched_norm_asks_its_consumers_for_their_lane():
             lins[0](act)
     finally:
         DynamicLinear.prof = old
+
+
+def test_scratch_lookup_rules(monkeypatch):
+    """Scratch buffers of the Python layer (host logic, no GPU): one pair per (device, stream handle); a Scratch that
+    is active in the thread replaces them whatever the stream; nothing is created while the stream is capturing;
+    release forgets one stream's pair."""
+    import torch
+    from kairos_amd import ops
+    made = []
+
+    def fake_new(idx, nbytes, zero, what):
+        if capturing[0]:
+            return real_new(idx, nbytes, zero, what)
+        made.append((idx, nbytes, zero, what))
+        return ("buf", len(made))
+
+    real_new = ops._new_scratch
+    capturing = [False]
+    monkeypatch.setattr(ops, "_new_scratch", fake_new)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: capturing[0])
+    monkeypatch.setattr(ops, "_workspaces", {})
+    monkeypatch.setattr(ops, "_gemv_workspaces", {})
+    a = ops.workspace_for("cuda:0", stream=111)
+    assert ops.workspace_for("cuda:0", stream=111) is a and ops.workspace_for("cuda:0", stream=222) is not a
+    g = ops.gemv_workspace_for("cuda:0", stream=111)
+    assert g is not a and made[-1][2] is True and made[0][2] is False          # the small-M scratch is created zeroed
+    # a stream handle that comes back after its stream was destroyed finds the same buffer (documented), until released
+    ops.release_workspace("cuda:0", stream=111)
+    assert ops.workspace_for("cuda:0", stream=111) is not a
+    # an active Scratch wins over the per-stream buffers, on any stream, and nests
+    outer, inner = ops.Scratch.__new__(ops.Scratch), ops.Scratch.__new__(ops.Scratch)
+    outer.gemm, outer.gemv, inner.gemm, inner.gemv = "og", "ov", "ig", "iv"
+    with outer:
+        assert ops.workspace_for("cuda:0", stream=333) == "og" and ops.gemv_workspace_for("cuda:0", stream=444) == "ov"
+        with inner:
+            assert ops.workspace_for("cuda:0", stream=333) == "ig"
+        assert ops.gemv_workspace_for("cuda:0", stream=111) == "ov"
+    assert ops.workspace_for("cuda:0", stream=222) not in ("og", "ig")
+    # during capture: existing buffers are handed out, missing ones are refused with the remedy
+    capturing[0] = True
+    assert ops.workspace_for("cuda:0", stream=222) is not None
+    with pytest.raises(RuntimeError, match="ensure_workspace"):
+        ops.workspace_for("cuda:0", stream=999)
+    with pytest.raises(RuntimeError, match="Scratch"):
+        ops.gemv_workspace_for("cuda:0", stream=999)
+    with outer:
+        assert ops.gemv_workspace_for("cuda:0", stream=999) == "ov"            # a graph that owns its scratch needs none
