@@ -236,6 +236,8 @@ def main():
                     help="counter runs: after set-up, run only the calls of the step that are booked under this kernel "
                          "label (e.g. 'gemm_w8a8[256]'), --steps times, and exit without the JSON line")
     ap.add_argument("--calls-json", default=None, help="with --only-label: where to write the number of calls made")
+    ap.add_argument("--group-m", type=int, default=0,
+                    help="experiments: tile rows per group of the GEMM kernels' tile order (0 = the library's default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on one GPU (every linear is independent and would shard by columns "
@@ -254,6 +256,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     names = {v: k for k, v in COMP_TYPE_NAME.items()}
+    if args.group_m:
+        ops.force_gemm_group_m(args.group_m)
 
     if args.resident_cache_mb > 0:
         from kairos_amd.temp_cache import ResidentCache, set_default_cache

@@ -276,9 +276,13 @@ int kmi_gemm_splits_for(int lane, int M, int N, int K, size_t workspace_bytes);
  * kmi_gemm_force_tile: 64, 128, 256, or 192 (W8A8 and fp16 operand-copy lanes only: 256 rows x 128 columns, two
  *   workgroups per CU); for kmi_gemm_w4a16 also 1032 / 1064 / 1128 (small-M variant, two wave quartets per
  *   workgroup) and 2032 / 2064 / 2128 (one).
- * kmi_gemm_force_splits: the number of K splits (needs a workspace in the call). */
+ * kmi_gemm_force_splits: the number of K splits (needs a workspace in the call).
+ * kmi_gemm_force_group_m: tile rows per group of the workgroup -> tile order of the GEMM kernels (every XCD takes a
+ *   contiguous run of a sequence that walks the tiles column-major in groups of that many tile rows; default 8); it
+ *   changes which tiles share an XCD's L2, never a result. */
 void kmi_gemm_force_tile(int tile);
 void kmi_gemm_force_splits(int splits);
+void kmi_gemm_force_group_m(int group_m);
 
 /* ---- interval lookup table (host only) --------------------------------------------------------- */
 

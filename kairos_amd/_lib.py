@@ -52,6 +52,7 @@ SIGNATURES = {
     "kmi_gemm_w4a16_wp_rows": [_I, _I, _I],
     "kmi_gemm_splits_for": [_I, _I, _I, _I, _Z],
     "kmi_gemm_force_splits": [_I],
+    "kmi_gemm_force_group_m": [_I],
     "kmi_lut_new": [],
     "kmi_lut_free": [_P],
     "kmi_lut_record": [_P, _I, _I],
@@ -69,7 +70,7 @@ SIGNATURES = {
 }
 _RESTYPE = {"kmi_get_last_error_string": ctypes.c_char_p, "kmi_lut_new": _P, "kmi_lut_free": None,
             "kmi_cache_create": _P, "kmi_cache_destroy": None,
-            "kmi_gemm_force_tile": None, "kmi_gemm_force_splits": None}
+            "kmi_gemm_force_tile": None, "kmi_gemm_force_splits": None, "kmi_gemm_force_group_m": None}
 
 _lib = None
 

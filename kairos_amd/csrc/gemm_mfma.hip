@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     int tm, tn;
     const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + BN - 1) / BN;
     const int split = blockIdx.x / (TM_ * TN_);
-    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn, p.group_m);
     const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
     const long a_row_bytes = I8 ? (long)K : (long)K * 2;
     const int KT_all = (int)(a_row_bytes >> 7);
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
     const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + 127) / 128;
     const int split = blockIdx.x / (TM_ * TN_);
     int tm, tn;
-    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn, p.group_m);
     const int m0 = tm * BM, n0 = p.n_begin + tn * 128;
     const int KT_all = K >> 6;                       // 64-wide k-tiles
     const int kt_per = (((KT_all + p.splits - 1) / p.splits) + KH - 1) / KH * KH;
@@ -592,7 +592,7 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
     auto setup = [&](int vb, Unit& u) {
         int tm, tn;
         u.split = vb / (TM_ * TN_);
-        tile_of_block(vb - u.split * (TM_ * TN_), TM_, TN_, tm, tn);
+        tile_of_block(vb - u.split * (TM_ * TN_), TM_, TN_, tm, tn, p.group_m);
         u.m0 = tm * BM;
         u.n0 = p.n_begin + tn * BN;
         u.t0 = u.split * t_per;                              // this unit covers stages t0 .. t0+T-1
@@ -832,6 +832,7 @@ static int cu_count() {
 template <int KIND, int BM, int BN, bool TILED, int NS_ = 4>
 static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
+    a.group_m = kmi_forced_group_m();
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const bool whole = (a.n_begin == 0 && a.n_cols == a.N);
@@ -884,6 +885,7 @@ static int launch_gemm(const GemmArgs& a_in, const Workspace& ws, hipStream_t st
 template <int BM, int KH = 2>
 static int launch_w4a16_wp(const GemmArgs& a_in, const Workspace& ws, hipStream_t st) {
     GemmArgs a = a_in;
+    a.group_m = kmi_forced_group_m();
     constexpr int PF = 4;                                        // k-tiles in flight per wave (8 measured 3-5 % slower at 32 / 64 rows)
     constexpr size_t lds = (size_t)KH * (PF + 1) * BM * 128;
     static_assert(lds <= 160 * 1024, "the activation ring must fit the LDS of a CU");
@@ -1053,6 +1055,9 @@ int kmi_gemm_args_check(const char* fn, const GemmArgs& a, bool tiled) {
 static thread_local int g_force_tile = 0;
 extern "C" void kmi_gemm_force_tile(int tile) { g_force_tile = tile; }
 int kmi_forced_tile() { return g_force_tile; }
+static thread_local int g_force_group_m = 0;
+extern "C" void kmi_gemm_force_group_m(int group_m) { g_force_group_m = group_m; }
+int kmi_forced_group_m() { return g_force_group_m; }
 
 int kmi_workspace_check(const char* fn, const void* workspace, size_t bytes, Workspace& ws) {
     if (workspace && !kmi_aligned16(workspace)) return kmi_set_error(KMI_E_ALIGN, "%s: workspace must be 16-byte aligned", fn);

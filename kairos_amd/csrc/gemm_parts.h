@@ -19,6 +19,7 @@ struct GemmArgs {
     void* partial;            // split-K: [splits][M][N] fp32 / int32 partial sums, else null
     int splits;               // number of K splits (1 = none)
     int n_begin, n_cols;      // output columns this launch covers (a multiple of the tile width unless it ends at N)
+    int group_m;              // tile rows per column-major group of the workgroup -> tile order (0 = the default, 8)
 };
 
 
@@ -315,8 +316,9 @@ __device__ __forceinline__ void sched_interleave() {
 // with a private L2.  Give every XCD a contiguous run of the tile sequence, and order that sequence
 // in column-major groups of GROUP_M tile rows, so the tiles resident on one XCD at a time form a
 // compact block that shares A row-panels and B column-panels in that XCD's L2.
-__device__ __forceinline__ void tile_of_block(int wg, int TM, int TN, int& tm, int& tn) {
-    constexpr int XCDS = 8, GROUP_M = 8;
+__device__ __forceinline__ void tile_of_block(int wg, int TM, int TN, int& tm, int& tn, int group_m = 0) {
+    constexpr int XCDS = 8;
+    const int GROUP_M = group_m > 0 ? group_m : 8;
     const int total = TM * TN;
     const int xcd = wg % XCDS, q = wg / XCDS;
     const int base = total / XCDS, rem = total % XCDS;
@@ -338,3 +340,4 @@ int kmi_gemm_args_check(const char* fn, const GemmArgs& a, bool tiled);
 int kmi_workspace_check(const char* fn, const void* workspace, size_t bytes, Workspace& ws);
 int kmi_pick_tile_rows(int M, int N, long row_bytes);
 int kmi_forced_tile();       // test hook of the calling thread, 0 = automatic
+int kmi_forced_group_m();    // test hook of the calling thread, 0 = the default tile order

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     int tm, tn;
     const int TM_ = (M + BM - 1) / BM, TN_ = (p.n_cols + BN - 1) / BN;
     const int split = blockIdx.x / (TM_ * TN_);
-    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn);
+    tile_of_block(blockIdx.x - split * (TM_ * TN_), TM_, TN_, tm, tn, p.group_m);
     const int m0 = tm * BM, n0 = p.n_begin + tn * BN;
     const int T_all = K >> 6;                                // 64-byte stages along K (K % 128 == 0: even)
     const int t_per = (((T_all + p.splits - 1) / p.splits) + 2 * KH - 1) / (2 * KH) * (2 * KH);   // whole groups per split and quartet
@@ -430,6 +430,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
 static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
+    a.group_m = kmi_forced_group_m();
     a.n_begin = n_begin;
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const Workspace ws = (a.n_begin == 0 && a.n_cols == a.N) ? ws_in : Workspace{nullptr, 0};   // column ranges: no split over K

@@ -482,6 +482,11 @@ def force_gemm_splits(splits):
     _lib.load().kmi_gemm_force_splits(int(splits))
 
 
+def force_gemm_group_m(group_m):
+    """Test hook of the calling thread: tile rows per group of the GEMM kernels' workgroup -> tile order (0 = default)."""
+    _lib.load().kmi_gemm_force_group_m(int(group_m))
+
+
 def force_gemm_tile(tile):
     """Test hook of the calling thread: 0 = automatic, else 64 / 128 / 192 / 256 (and the 1xxx / 2xxx selectors of the
     small-M W4A16 variant)."""
