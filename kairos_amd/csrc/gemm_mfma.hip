@@ -556,6 +556,13 @@ __global__ __launch_bounds__(256 * KH) void gemm_w4a16_wp_kernel(GemmArgs p) {
 // fetches the chunk that belongs in slot l.  The tiled weight layout ([N/128][K-stages][128][64 B],
 // already swizzled) makes the B side a straight 8 KiB copy per 128-row strip.
 
+// Wait until at most KEEP direct loads of this thread are outstanding, then meet the other waves.
+// A plain barrier instruction (no fence): the fence of __syncthreads would drain every load.
+template <int KEEP>
+__device__ __forceinline__ void direct_stage_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(KEEP) : "memory");
+}
+
 template <int KIND, int BM, int BN, bool TILED_B, int NS, bool PERSIST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((NS == 3 && BM == 256 && BN == 128) ? 2 : 1)))
 void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for two workgroups per CU: <= 256 registers, 72 KiB of LDS
@@ -671,41 +678,60 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
 #pragma unroll
         for (int j = 0; j < FN; ++j) fb[set][j] = *reinterpret_cast<const u4_t*>(st + off_b[s] + j * 2048);
     };
-    auto mfma_step = [&](int set) {
+    // `fresh`: the tile's first k-step, which starts from a zero operand instead of cleared accumulators
+    auto mfma_step = [&](int set, auto fresh) {
+        constexpr bool FRESH = decltype(fresh)::value;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
+                const acc_t c = FRESH ? acc_t{} : acc[i][j];
                 if constexpr (I8)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i4_t, fb[set][j]),
-                                                                      __builtin_bit_cast(i4_t, fa[set][i]), acc[i][j], 0, 0, 0);
+                                                                      __builtin_bit_cast(i4_t, fa[set][i]), c, 0, 0, 0);
                 else
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, fb[set][j]),
-                                                                       __builtin_bit_cast(h8_t, fa[set][i]), acc[i][j], 0, 0, 0);
+                                                                       __builtin_bit_cast(h8_t, fa[set][i]), c, 0, 0, 0);
             }
     };
     constexpr int NMF = FM * FN, NRD = FM + FN;
 
-    // Wait until at most `keep` direct loads of this thread are outstanding, then meet the other waves.
-    // A plain barrier instruction (no fence): the fence of __syncthreads would drain every load.
-#define KMI_STAGE_BARRIER(keep) asm volatile("s_waitcnt vmcnt(" #keep ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
-
     // ---- pipeline: stage t is computed while stages t+1 .. t+NS-1 are in flight.  Every MFMA block
     // (one k-step) issues, between its first MFMAs, the fragment reads of the NEXT k-step into the
     // other register set, so LDS latency hides behind the block and nothing is read after it.
-#define KMI_STAGE_WAIT()                                                   \
-    do {                                                                   \
-        if constexpr (NLD * (NS - 2) == 16) KMI_STAGE_BARRIER(16);         \
-        else if constexpr (NLD * (NS - 2) == 14) KMI_STAGE_BARRIER(14);    \
-        else if constexpr (NLD * (NS - 2) == 8) KMI_STAGE_BARRIER(8);      \
-        else if constexpr (NLD * (NS - 2) == 6) KMI_STAGE_BARRIER(6);      \
-        else if constexpr (NLD * (NS - 2) == 4) KMI_STAGE_BARRIER(4);      \
-        else if constexpr (NLD * (NS - 2) == 3) KMI_STAGE_BARRIER(3);      \
-        else KMI_STAGE_BARRIER(0);                                         \
-    } while (0)
-    static_assert(NS == 4 || NS == 3, "vmcnt immediates above assume 3 or 4 stages");
-    static_assert(NLD * (NS - 2) == 16 || NLD * (NS - 2) == 14 || NLD * (NS - 2) == 8 || NLD * (NS - 2) == 6 || NLD * (NS - 2) == 4 ||
-                  NLD * (NS - 2) == 3, "no wait immediate for this tile and depth");
+    // Between the two blocks of a stage the wave waits until stage t+1 has landed (at most `keep` younger direct
+    // loads of this thread outstanding: loads retire in issue order) and meets the other waves; see
+    // direct_stage_barrier.  One iteration, `left` = stages after t, known at compile time when below NS:
+    // the last NS iterations issue only loads that exist and wait for exactly what is still on its way.
+    static_assert(NS == 4 || NS == 3, "three or four stages");
+    static_assert(NLD * (NS - 2) <= 48, "wait immediates stay well below the counter's range");
+    using Yes = std::integral_constant<bool, true>;
+    using I0 = std::integral_constant<int, 0>;
+    using No = std::integral_constant<bool, false>;
+    auto stage_body = [&](const Unit& u, int t, auto fresh, auto left_, auto extra_, auto&& after_last_load) {
+        constexpr int LEFT = decltype(left_)::value;            // NS stands for "NS or more"
+        constexpr int EXTRA = decltype(extra_)::value;          // other loads of this thread, younger than every stage load
+        constexpr bool LD1 = LEFT >= NS - 1, LD0 = LEFT >= NS;   // stages t+NS-1 and t+NS exist
+        constexpr int YOUNGER = LEFT - 1 < NS - 2 ? LEFT - 1 : NS - 2;   // whole stages issued after stage t+1
+        // Slot (t-1) % NS was released by the previous barrier: it takes k-stage t+NS-1, half of the
+        // loads in each of the two MFMA blocks that follow that barrier, so the memory pipe sees one
+        // load per wave every few MFMAs instead of a burst.
+        read_frags(t, 1, 1);
+        if constexpr (LD1) issue_half(u, t + NS - 1, 1);
+        if constexpr (LEFT == NS - 1) after_last_load();         // the last stage load of the unit is out
+        mfma_step(0, fresh);                                     // (t, step 0)
+        sched_interleave<NMF, NRD, 0, LD1 ? NLD - NLD0 : 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (LEFT >= 1) {
+            // stage t+1 has landed for every wave and stage t is fully in registers
+            direct_stage_barrier<NLD * YOUNGER + EXTRA>();
+            read_frags(t + 1, 0, 0);
+        }
+        if constexpr (LD0) issue_half(u, t + NS, 0);
+        mfma_step(1, No{});                                      // (t, step 1)
+        sched_interleave<NMF, LEFT >= 1 ? NRD : 0, 0, LD0 ? NLD0 : 0>();
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // The epilogue's per-wave patches: the start of LDS in the one-tile form; the END of LDS in the
     // persistent form (stage 3 and the last KiB of stage 2), which leaves stages 0 and 1 free to receive
     // the next unit's first k-stages while this unit's results are written out.
@@ -715,12 +741,8 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
 
     bool ahead = false;                                      // stages 0 and 1 of `cur` are already on their way
     for (int vb = blockIdx.x;;) {
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+        // Stages past the end of a short K range (fewer than NS-1 stages) are clamped reloads into free slots; the
+        // waits of the last iterations then cover them too, which is harmless.
         if (PERSIST && ahead) {
             // every wave has left the previous epilogue before stage 2 (whose end holds a patch) is refilled
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -731,56 +753,78 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
             for (int t = 0; t < NS - 1; ++t) issue_stage(cur, t);
         }
         // loads retire in issue order and the stores of a previous epilogue are older than every load
-        // counted here, so the same immediates hold for the first and for later units
-        KMI_STAGE_WAIT();
-        issue_half(cur, NS - 1, 0);
+        // counted here, so the same immediate holds for the first and for later units
+        direct_stage_barrier<NLD * (NS - 2)>();
+        if (cur.T >= NS) issue_half(cur, NS - 1, 0);
         read_frags(0, 0, 0);
-        for (int t = 0; t < cur.T; ++t) {
-            // Slot (t-1) % NS was released by the previous barrier: it takes k-stage t+NS-1, half of the
-            // loads in each of the two MFMA blocks that follow that barrier, so the memory pipe sees one
-            // load per wave every few MFMAs instead of a burst.
-            read_frags(t, 1, 1);
-            issue_half(cur, t + NS - 1, 1);
-            mfma_step(0);                                    // (t, step 0)
-            sched_interleave<NMF, NRD, 0, NLD - NLD0>();
-            __builtin_amdgcn_sched_barrier(0);
-            // stage t+1 has landed for every wave and stage t is fully in registers
-            KMI_STAGE_WAIT();
-            read_frags(t + 1, 0, 0);                         // past the last stage: a harmless re-read
-            issue_half(cur, t + NS, 0);
-            mfma_step(1);                                    // (t, step 1)
-            sched_interleave<NMF, NRD, 0, NLD0>();
-            __builtin_amdgcn_sched_barrier(0);
+        int t = 0;
+        if (cur.T > NS) {
+            stage_body(cur, 0, Yes{}, std::integral_constant<int, NS>{}, I0{}, NoHook{});
+            t = 1;
+        } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+        }
+        for (; t + NS < cur.T; ++t) stage_body(cur, t, No{}, std::integral_constant<int, NS>{}, I0{}, NoHook{});
+        // W8A8: this lane's row and column factors travel under the last stages: FM + FN two-byte loads, issued right
+        // behind the unit's last stage load, so they are the youngest loads of the thread and the waits below make
+        // room for exactly them.
+        constexpr int NF = (KIND == KIND_W8A8) ? FM + FN : 0;
+        EpiFactors<FM, FN> fac;
+        auto load_factors = [&]() {
+            if constexpr (KIND == KIND_W8A8) {
+                asm volatile("" ::: "memory");
+                epilogue_factors<BM, BN, FM, FN>(p, cur.m0, cur.n0, wave, lane, fac);
+                asm volatile("" ::: "memory");
+            }
+        };
+        if (cur.T < NS) load_factors();                          // no iteration below issues a stage load
+        static_for<0, NS>([&](auto back) {                       // left = NS-1 .. 0
+            constexpr int LEFT = NS - 1 - decltype(back)::value;
+            if (t < cur.T && cur.T - 1 - t == LEFT) {
+                stage_body(cur, t, No{}, std::integral_constant<int, LEFT>{}, std::integral_constant<int, NF>{}, load_factors);
+                ++t;
+            }
+        });
+
+        Unit nxt;
+        bool more = false;
+        if constexpr (PERSIST) {                                 // under the last MFMAs and whatever a short K left in flight
+            more = vb + (int)gridDim.x < nvirt;
+            if (more) setup(vb + (int)gridDim.x, nxt);
         }
         // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
         if constexpr (PERSIST) {
             // the host uses this form without a split over K only
-            Unit nxt;
-            const bool more = vb + (int)gridDim.x < nvirt;
-            if (more) setup(vb + (int)gridDim.x, nxt);
             auto start_next = [&]() {
                 if (more) {
                     issue_stage(nxt, 0);
                     issue_stage(nxt, 1);
                 }
             };
-            if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next);
-            else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next);
+            const EpiFactors<FM, FN>* pre = (KIND == KIND_W8A8) ? &fac : nullptr;
+            if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next, pre);
+            else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem + PATCH_OFF, cur.m0, cur.n0, wave, lane, start_next, pre);
             if (!more) break;
             cur = nxt;
             ahead = true;
             vb += (int)gridDim.x;
         } else {
             if (p.splits > 1) store_partial<BM, BN, FM, FN>(p, acc, cur.split, cur.m0, cur.n0, wave, lane);
-            else if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane);
-            else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane);
+            else {
+                const EpiFactors<FM, FN>* pre = (KIND == KIND_W8A8) ? &fac : nullptr;
+                if (p.bias) gemm_epilogue<KIND, BM, BN, true, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane, NoHook{}, pre);
+                else gemm_epilogue<KIND, BM, BN, false, FM, FN>(p, acc, smem, cur.m0, cur.n0, wave, lane, NoHook{}, pre);
+            }
             break;
         }
     }
-#undef KMI_STAGE_WAIT
-#undef KMI_STAGE_BARRIER
 #endif
 }
 

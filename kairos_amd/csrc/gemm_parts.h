@@ -125,20 +125,57 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
     }
 }
 
-// Epilogue shared by both kernels.  The MFMAs are issued with the weight fragment as the first
+// Epilogue shared by the GEMM kernels.  The MFMAs are issued with the weight fragment as the first
 // operand, so an accumulator tile is D^T: lane (c = lane&31, hl = lane>>5) holds, for activation row
 // m = c, the output columns n = 8g + 4hl + r (e = 4g + r) -- four consecutive columns per g.
 // A wave converts one 32-row block at a time, writes it to its private LDS patch as fp16 [32][BN/2]
 // (8-byte writes, pitch padded by 8 bytes -> conflict free), and streams it out with 16-byte stores
 // in which 16 consecutive lanes cover 256 contiguous bytes of one output row.
+//
+// With one wave per SIMD every instruction of the epilogue, scalar or vector, costs an issue slot that nothing
+// else fills, so the instruction count is the cost.  Three things keep it down:
+//   * W8A8: the factor of element (m, n) is wscale[n] * ascale[m], exact in fp32 (two 11-bit significands).  One
+//     32x32x8 fp16 MFMA per accumulator tile, fed with the wave's 32 column factors and 32 row factors in its k = 0
+//     slice and zeros elsewhere, writes those 1024 products in the accumulator's own lane layout; the matrix pipe is
+//     idle here anyway.  Element work is then read, int -> float, one multiply, pack.
+//   * a tile that lies inside the matrix stores through a buffer resource at the tile's origin: a per-lane
+//     offset fixed for the kernel, a scalar offset per store, no masks and no 64-bit address arithmetic;
+//   * accumulators are read four at a time, so no read is followed by its own use (a wait state otherwise).
 struct NoHook {
     __device__ __forceinline__ void operator()() const {}
 };
+
+// This lane's entries of the per-column and per-row factors of a W8A8 tile: ws[j] belongs to column
+// nw + 32j + lane%32 of the wave's block, as[i] to row mw + 32i + lane%32.
+template <int FM, int FN>
+struct EpiFactors {
+    half_t ws[FN];
+    half_t as[FM];
+};
+template <int BM, int BN, int FM, int FN>
+__device__ __forceinline__ void epilogue_factors(const GemmArgs& p, int m0, int n0, int wave, int lane, EpiFactors<FM, FN>& f) {
+    const int c = lane & 31;
+    const int mw = m0 + (wave >> 1) * (BM / 2) + c, nw = n0 + (wave & 1) * (BN / 2) + c;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int n = nw + j * 32;
+        f.ws[j] = p.wscales[n < p.N ? n : p.N - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = mw + i * 32;
+        f.as[i] = p.ascales[m < p.M ? m : p.M - 1];
+    }
+}
+
 // `after_loads` runs once the per-column and per-row factors have arrived and before the first result leaves: a
 // persistent kernel starts the next tile's operand loads there, behind every load this epilogue waits for.
+// `pre`: W8A8 factors the caller loaded ahead of time (else they are loaded here).
 template <int KIND, int BM, int BN, bool HAS_BIAS, int FM, int FN, typename acc_t, typename Hook = NoHook>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM][FN], char* smem, int m0, int n0,
-                                              int wave, int lane, Hook after_loads = Hook{}) {
+                                              int wave, int lane, Hook after_loads = Hook{},
+                                              const EpiFactors<FM, FN>* pre = nullptr
+                                              ) {
     const int M = p.M, N = p.N;
     const int wm = wave >> 1, wn = wave & 1;
     const int c = lane & 31, hl = lane >> 5;
@@ -157,6 +194,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 }
         }
     } else {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass knows neither the buffer resource type nor the MFMA
         constexpr int WN = BN / 2;                       // columns per wave
         constexpr bool BIG = FM * FN >= 12;              // accumulators in AGPRs, read explicitly
         constexpr int PITCH = WN * 2 + 8;                // bytes
@@ -172,12 +210,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
             for (int g = 0; g < 4; ++g) {
                 int n = nw + j * 32 + 8 * g + 4 * hl;
                 n = n < N ? n : N - 4;
-                if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) ws4[j][g] = *reinterpret_cast<const h4_t*>(p.wscales + n);
+                if constexpr (KIND == KIND_W8A16) ws4[j][g] = *reinterpret_cast<const h4_t*>(p.wscales + n);
                 if constexpr (HAS_BIAS) bs4[j][g] = *reinterpret_cast<const h4_t*>(p.bias + n);
             }
         float wsf[FN][4][4];                              // fp32 once, not once per row block
         (void)wsf;
-        if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) {
+        if constexpr (KIND == KIND_W8A16) {
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
@@ -185,31 +223,43 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
 #pragma unroll
                     for (int r = 0; r < 4; ++r) wsf[j][g][r] = (float)ws4[j][g][r];
         }
-        float as_i[FM];
-        (void)as_i;
+        // W8A8: the operands of the factor tiles.  Weight side first, as in the main loop, so the product tile has
+        // the accumulators' layout; only the k = 0..3 slice (lanes 0..31) carries a value, in its first element.
+        h4_t wop[FN], aop[FM];
+        (void)wop; (void)aop;
         if constexpr (KIND == KIND_W8A8) {
+            EpiFactors<FM, FN> f;
+            if (pre) f = *pre;
+            else epilogue_factors<BM, BN, FM, FN>(p, m0, n0, wave, lane, f);
+            const half_t zero = (half_t)0.f;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const int m = mw + i * 32 + c;
-                as_i[i] = (float)p.ascales[m < M ? m : M - 1];
-            }
+            for (int j = 0; j < FN; ++j) wop[j] = h4_t{hl == 0 ? f.ws[j] : zero, zero, zero, zero};
+#pragma unroll
+            for (int i = 0; i < FM; ++i) aop[i] = h4_t{hl == 0 ? f.as[i] : zero, zero, zero, zero};
+            // built here, once: the statements that use them must find them in registers, not rebuild them on the spot
+#pragma unroll
+            for (int j = 0; j < FN; ++j) asm volatile("" : "+v"(wop[j]));
+#pragma unroll
+            for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(aop[i]));
         }
         if constexpr (!std::is_same<Hook, NoHook>::value) {
             // name every loaded factor as an operand, so the compiler places its waits for them here and
             // none of its later waits can fall behind the loads that the hook starts
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (KIND == KIND_W8A8) asm volatile("" : "+v"(wop[j]));
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    if constexpr (KIND == KIND_W8A16 || KIND == KIND_W8A8) {
+                    if constexpr (KIND == KIND_W8A16) {
 #pragma unroll
                         for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(wsf[j][g][r]));
                     }
                     if constexpr (HAS_BIAS) asm volatile("" : "+v"(bs4[j][g]));
                 }
+            }
             if constexpr (KIND == KIND_W8A8) {
 #pragma unroll
-                for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(as_i[i]));
+                for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(aop[i]));
             }
             asm volatile("" ::: "memory");
             after_loads();
@@ -217,33 +267,92 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         }
         half_t* outp = static_cast<half_t*>(p.out);
         const bool wide = (N & 7) == 0;                  // 16-byte row segments stay aligned
+        // a tile inside the matrix: stores relative to the tile's origin, 32-bit offsets (256 rows of N fp16)
+        const bool inside = wide && m0 + BM <= M && n0 + BN <= N && (64 % CPR) == 0;
+        const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(outp + ((long)m0 * N + n0), 0, -1, 0x00020000);
+        const uint32_t ovoff = (uint32_t)(((wm * (BM / 2) + lane / CPR) * N + wn * WN + (lane % CPR) * 8) * 2);
+        // Factor tiles, two in flight: tile t+1 is issued before tile t is converted.  Written as asm with a VGPR
+        // destination: the compiler would place the result in AGPRs, and every element would cost a read again.
+        // The compiler knows nothing of the latency of such a statement, so the distance between a product and its
+        // first use is built from ordered statements: the first tile carries its wait states itself; every later
+        // tile is handed to its users (`settled`) only behind the 64 multiplies of the tile before it, each a
+        // statement of its own, in program order: far more than the 19 wait states a 16-pass MFMA asks for.
+        f16_t fac[2];
+        (void)fac;
+        auto factor_tile = [&](int t) {
+            if constexpr (KIND == KIND_W8A8) {
+                if (t == 0)
+                    asm volatile("s_nop 3\n\tv_mfma_f32_32x32x8_f16 %0, %1, %2, 0\n\ts_nop 15\n\ts_nop 7"
+                                 : "=&v"(fac[0]) : "v"(wop[0]), "v"(aop[0]));
+                else if (t < FM * FN)   // the wait state in front: the compiler may have copied an operand just before
+                    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x8_f16 %0, %1, %2, 0" : "=&v"(fac[t & 1]) : "v"(wop[t % FN]), "v"(aop[t / FN]));
+            }
+        };
+        auto settled = [&](int t) {
+            if constexpr (KIND == KIND_W8A8) asm volatile("" : "+v"(fac[t & 1]));
+        };
+        factor_tile(0);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+            for (int j = 0; j < FN; ++j) {
+                settled(i * FN + j);
+                factor_tile(i * FN + j + 1);
+                if constexpr (KIND == KIND_W8A8 && BIG && !HAS_BIAS) {
+                    // One wave per SIMD: a dependent instruction issued right behind its producer waits about one
+                    // more issue slot, and nothing else fills it.  Eight elements at a time, every step a statement
+                    // of its own in the order written, keep producer and user at least four instructions apart.
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    half_t h[4];
+                    for (int gg = 0; gg < 2; ++gg) {
+                        int ai[8];
+                        float af[8], pr[8];
+                        uint32_t pk[4];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float v;
-                        const auto a = acc_elem<BIG>(acc[i][j][4 * g + r]);
-                        if constexpr (KIND == KIND_W8A8) {
-                            // product rounded to fp32 first, then to fp16 (two roundings, as the
-                            // reference epilogue): keep the compiler from fusing them into one
-                            v = (float)a * (wsf[j][g][r] * as_i[i]);
-                            asm volatile("" : "+v"(v));
-                        } else if constexpr (KIND == KIND_W8A16) {
-                            v = a * wsf[j][g][r];
-                        } else {
-                            v = a;
+                        for (int e = 0; e < 8; ++e) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ai[e]) : "a"(acc[i][j][8 * gg + e]));
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) asm volatile("v_cvt_f32_i32 %0, %1" : "=v"(af[e]) : "v"(ai[e]));
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float s = fac[(i * FN + j) & 1][8 * gg + e];
+                            asm volatile("v_mul_f32 %0, %1, %2" : "=v"(pr[e]) : "v"(af[e]), "v"(s));
                         }
-                        h[r] = (half_t)v;
-                        if constexpr (HAS_BIAS) h[r] = (half_t)((float)h[r] + (float)bs4[j][g][r]);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(pk[q]) : "v"(pr[2 * q]), "v"(pr[2 * q + 1]));
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            *reinterpret_cast<u2_t*>(patch + c * PITCH + (j * 32 + 8 * (2 * gg + h) + 4 * hl) * 2) = u2_t{pk[2 * h], pk[2 * h + 1]};
                     }
-                    h4_t pk = {h[0], h[1], h[2], h[3]};
-                    *reinterpret_cast<h4_t*>(patch + c * PITCH + (j * 32 + 8 * g + 4 * hl) * 2) = pk;
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        decltype(acc_elem<BIG>(acc[i][j][0])) a[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) a[r] = acc_elem<BIG>(acc[i][j][4 * g + r]);
+                        half_t h[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            float v;
+                            if constexpr (KIND == KIND_W8A8) {
+                                // product rounded to fp32 first, then to fp16 (two roundings, as the
+                                // reference epilogue): keep the compiler from fusing them into one
+                                // (the multiply is a statement of its own, which also makes it one of the ordered
+                                // instructions that stand between a factor tile and its users)
+                                const float s = fac[(i * FN + j) & 1][4 * g + r];
+                                const float fa = (float)a[r];
+                                asm volatile("v_mul_f32 %0, %1, %2" : "=v"(v) : "v"(fa), "v"(s));
+                            } else if constexpr (KIND == KIND_W8A16) {
+                                v = a[r] * wsf[j][g][r];
+                            } else {
+                                v = a[r];
+                            }
+                            h[r] = (half_t)v;
+                            if constexpr (HAS_BIAS) h[r] = (half_t)((float)h[r] + (float)bs4[j][g][r]);
+                        }
+                        h4_t pk = {h[0], h[1], h[2], h[3]};
+                        *reinterpret_cast<h4_t*>(patch + c * PITCH + (j * 32 + 8 * g + 4 * hl) * 2) = pk;
+                    }
                 }
+            }
             // the patch is private to the wave and LDS serves a wave's requests in order
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             constexpr int NK = 32 * CPR / 64;                // 16-byte chunks per lane and 32-row block
@@ -270,6 +379,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 continue;
             }
+            if (inside) {
+#pragma unroll
+                for (int k = 0; k < NK; ++k)
+                    __builtin_amdgcn_raw_buffer_store_b128(v[k], orsrc, ovoff, (uint32_t)((i * 32 + k * (64 / CPR)) * N * 2), 2 /* nt */);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
+                continue;
+            }
             const int n = nw + (lane % CPR) * 8;             // CPR divides 64: the column is the same for every k
             half_t* dst = outp + (long)(mw + i * 32 + lane / CPR) * N + n;
             if (wide) {
@@ -289,6 +405,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
         }
+#endif
     }
 }
 
