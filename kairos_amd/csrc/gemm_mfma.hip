@@ -758,7 +758,18 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
         if (cur.T >= NS) issue_half(cur, NS - 1, 0);
         read_frags(0, 0, 0);
         int t = 0;
+        Unit nxt;
+        bool more = false, nxt_ready = false;
         if (cur.T > NS) {
+            if constexpr (PERSIST) {
+                // the next unit's place and load offsets: integer work for the issue slots between the first MFMAs
+                // (no branch in it, so that it can be scheduled into the block: past the last unit it describes the
+                // last unit again and is not used)
+                const int nb = vb + (int)gridDim.x;
+                more = nb < nvirt;
+                setup(more ? nb : nvirt - 1, nxt);
+                nxt_ready = true;
+            }
             stage_body(cur, 0, Yes{}, std::integral_constant<int, NS>{}, I0{}, NoHook{});
             t = 1;
         } else {
@@ -791,21 +802,25 @@ void gemm_direct_kernel(GemmArgs p) {   // the 256 x 128 instance is built for t
             }
         });
 
-        Unit nxt;
-        bool more = false;
-        if constexpr (PERSIST) {                                 // under the last MFMAs and whatever a short K left in flight
-            more = vb + (int)gridDim.x < nvirt;
-            if (more) setup(vb + (int)gridDim.x, nxt);
+        if constexpr (PERSIST) {
+            if (!nxt_ready) {                                    // a short K range: no first iteration to hide it in
+                more = vb + (int)gridDim.x < nvirt;
+                if (more) setup(vb + (int)gridDim.x, nxt);
+            }
         }
         // no direct load may outlive the workgroup or land in LDS that the epilogue reuses
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
         if constexpr (PERSIST) {
             // the host uses this form without a split over K only
-            auto start_next = [&]() {
+            // stages 0 and 1 of the next unit, spread over the first three row blocks of this unit's epilogue; all of
+            // them are older than the last block's stores, which is what the wait at the top of the next unit counts on
+            static_assert(FM >= 4, "the next unit's first loads are dealt over three row blocks");
+            auto start_next = [&](int i) {
                 if (more) {
-                    issue_stage(nxt, 0);
-                    issue_stage(nxt, 1);
+                    if (i == 0) issue_stage(nxt, 0);
+                    else if (i == 1) issue_half(nxt, 1, 0);
+                    else if (i == 2) issue_half(nxt, 1, 1);
                 }
             };
             const EpiFactors<FM, FN>* pre = (KIND == KIND_W8A8) ? &fac : nullptr;

@@ -143,6 +143,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
 //   * accumulators are read four at a time, so no read is followed by its own use (a wait state otherwise).
 struct NoHook {
     __device__ __forceinline__ void operator()() const {}
+    __device__ __forceinline__ void operator()(int) const {}
 };
 
 // This lane's entries of the per-column and per-row factors of a W8A8 tile: ws[j] belongs to column
@@ -168,12 +169,14 @@ __device__ __forceinline__ void epilogue_factors(const GemmArgs& p, int m0, int 
     }
 }
 
-// `after_loads` runs once the per-column and per-row factors have arrived and before the first result leaves: a
-// persistent kernel starts the next tile's operand loads there, behind every load this epilogue waits for.
+// `before_block(i)` runs in front of the conversion of every 32-row block, the first time once the per-column and
+// per-row factors have arrived and before the first result leaves: a persistent kernel issues the next tile's first
+// operand loads there, a few per block (a burst of them would queue up in the address path while the wave waits),
+// behind every load this epilogue waits for.
 // `pre`: W8A8 factors the caller loaded ahead of time (else they are loaded here).
 template <int KIND, int BM, int BN, bool HAS_BIAS, int FM, int FN, typename acc_t, typename Hook = NoHook>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM][FN], char* smem, int m0, int n0,
-                                              int wave, int lane, Hook after_loads = Hook{},
+                                              int wave, int lane, Hook before_block = Hook{},
                                               const EpiFactors<FM, FN>* pre = nullptr
                                               ) {
     const int M = p.M, N = p.N;
@@ -262,8 +265,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                 for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(aop[i]));
             }
             asm volatile("" ::: "memory");
-            after_loads();
-            asm volatile("" ::: "memory");
         }
         half_t* outp = static_cast<half_t*>(p.out);
         const bool wide = (N & 7) == 0;                  // 16-byte row segments stay aligned
@@ -294,6 +295,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         factor_tile(0);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
+            if constexpr (!std::is_same<Hook, NoHook>::value) {
+                before_block(i);
+                asm volatile("" ::: "memory");
+            }
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 settled(i * FN + j);
