@@ -292,6 +292,59 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         auto settled = [&](int t) {
             if constexpr (KIND == KIND_W8A8) asm volatile("" : "+v"(fac[t & 1]));
         };
+        // A row block leaves in two steps, one block apart: its 16-byte chunks are read back from the patch right
+        // behind its last write, and stored while the next block is being converted (after that block's first tile),
+        // so neither the LDS round trip nor the store issue stands between two conversions.
+        constexpr int NK = 32 * CPR / 64;                    // 16-byte chunks per lane and 32-row block
+        static_assert((32 * CPR) % 64 == 0, "whole 16-byte chunks per lane");
+        u4_t v[NK];
+        auto read_block = [&]() {
+#pragma unroll
+            for (int k = 0; k < NK; ++k) {
+                const int idx = k * 64 + lane;
+                v[k] = *reinterpret_cast<const u4_t*>(patch + (idx / CPR) * PITCH + (idx % CPR) * 16);
+            }
+        };
+        auto store_block = [&](int i) {
+            if constexpr (64 % CPR != 0) {                   // 96 columns per wave: the column changes with k
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int idx = k * 64 + lane;
+                    const int m = mw + i * 32 + idx / CPR, n = nw + (idx % CPR) * 8;
+                    half_t* d = outp + (long)m * N + n;
+                    if (wide) {
+                        if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(d));
+                    } else {
+                        if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
+                        if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
+                    }
+                }
+                return;
+            }
+            if (inside) {
+#pragma unroll
+                for (int k = 0; k < NK; ++k)
+                    __builtin_amdgcn_raw_buffer_store_b128(v[k], orsrc, ovoff, (uint32_t)((i * 32 + k * (64 / CPR)) * N * 2), 2 /* nt */);
+                return;
+            }
+            const int n = nw + (lane % CPR) * 8;             // CPR divides 64: the column is the same for every k
+            half_t* dst = outp + (long)(mw + i * 32 + lane / CPR) * N + n;
+            if (wide) {
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
+                    if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N));
+                }
+            } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
+                    half_t* d = dst + (long)k * (64 / CPR) * N;
+                    if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
+                    if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
+                }
+            }
+        };
         factor_tile(0);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
@@ -301,6 +354,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
             }
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
+                if (j == (FN > 1 ? 1 : 0) && i > 0) {         // the block before: its chunks have arrived by now
+                    store_block(i - 1);
+                    asm volatile("" ::: "memory");
+                }
                 settled(i * FN + j);
                 factor_tile(i * FN + j + 1);
                 if constexpr (KIND == KIND_W8A8 && BIG && !HAS_BIAS) {
@@ -358,58 +415,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
                     }
                 }
             }
-            // the patch is private to the wave and LDS serves a wave's requests in order
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            constexpr int NK = 32 * CPR / 64;                // 16-byte chunks per lane and 32-row block
-            u4_t v[NK];
-#pragma unroll
-            for (int k = 0; k < NK; ++k) {                   // all reads first: one LDS round trip, not NK
-                const int idx = k * 64 + lane;
-                v[k] = *reinterpret_cast<const u4_t*>(patch + (idx / CPR) * PITCH + (idx % CPR) * 16);
-            }
-            if constexpr (64 % CPR != 0) {                   // 96 columns per wave: the column changes with k
-                static_assert((32 * CPR) % 64 == 0, "whole 16-byte chunks per lane");
-#pragma unroll
-                for (int k = 0; k < NK; ++k) {
-                    const int idx = k * 64 + lane;
-                    const int m = mw + i * 32 + idx / CPR, n = nw + (idx % CPR) * 8;
-                    half_t* d = outp + (long)m * N + n;
-                    if (wide) {
-                        if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(d));
-                    } else {
-                        if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
-                        if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
-                    }
-                }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                continue;
-            }
-            if (inside) {
-#pragma unroll
-                for (int k = 0; k < NK; ++k)
-                    __builtin_amdgcn_raw_buffer_store_b128(v[k], orsrc, ovoff, (uint32_t)((i * 32 + k * (64 / CPR)) * N * 2), 2 /* nt */);
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
-                continue;
-            }
-            const int n = nw + (lane % CPR) * 8;             // CPR divides 64: the column is the same for every k
-            half_t* dst = outp + (long)(mw + i * 32 + lane / CPR) * N + n;
-            if (wide) {
-#pragma unroll
-                for (int k = 0; k < NK; ++k) {
-                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
-                    if (m < M && n < N) __builtin_nontemporal_store(v[k], reinterpret_cast<u4_t*>(dst + (long)k * (64 / CPR) * N));
-                }
-            } else {                                         // N % 8 == 4: two 8-byte halves, each whole or absent
-#pragma unroll
-                for (int k = 0; k < NK; ++k) {
-                    const int m = mw + i * 32 + (k * 64 + lane) / CPR;
-                    half_t* d = dst + (long)k * (64 / CPR) * N;
-                    if (m < M && n < N) *reinterpret_cast<u2_t*>(d) = u2_t{v[k][0], v[k][1]};
-                    if (m < M && n + 4 < N) *reinterpret_cast<u2_t*>(d + 4) = u2_t{v[k][2], v[k][3]};
-                }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // reads done before the patch is rewritten
+            // The patch is private to the wave and LDS serves a wave's requests in order: these reads see the writes
+            // above without a wait, and the next block's writes cannot overtake them.
+            asm volatile("" ::: "memory");
+            read_block();
         }
+        store_block(FM - 1);
 #endif
     }
 }
