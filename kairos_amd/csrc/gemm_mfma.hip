@@ -1006,7 +1006,10 @@ static int pick_tile(int M, int N, long row_bytes) {
         // One round either way: 256 x 192 tiles (N a multiple of 192 and of the 128-row weight strips; selector 320,
         // tiled weights only) put the same output on more CUs with less work each.  The narrower tile is less efficient
         // per MFMA, so the gain is small: 2048 x 6144 x 4096 51.9 against 54.9 us, 2048 x 4608 x 3584 37.9 against 45.1.
-        if (split == 1 && N % 384 == 0 && wgs(256, 192) <= 256 && wgs(256, 256) < wgs(256, 192)) return 320;
+        // The same holds for whole rounds of them where the wider tile leaves a ragged one (4096 x 6144 x 4096: two
+        // rounds, 88.1 against 93.7 us for 1.5 rounds of 256 x 256 with a 128 x 128 tail).
+        const long w192 = wgs(256, 192), w256 = wgs(256, 256);
+        if (split == 1 && N % 384 == 0 && w256 < w192 && (w192 <= 256 || (w192 % 256 == 0 && w256 % 256 != 0))) return 320;
         return 256;
     }
     // too few 256 x 256 tiles for the CUs, yet the rows are too short to split: 256 x 128 tiles, two workgroups per CU
