@@ -3,7 +3,9 @@
 // small-M W4A16 kernel and nothing else).  No product path calls them; `python -m kairos_amd.bench_extra floor` does.
 #include "kmi_common.h"
 
-static __device__ uint32_t g_probe_sink;
+// volatile and with external linkage: a sink that nothing reads would let the compiler drop the stores to it, and with them
+// every load of the probes
+__device__ volatile uint32_t g_probe_sink;
 
 __global__ void probe_empty_kernel() {
     if (threadIdx.x == 9999) g_probe_sink = 1;

@@ -302,6 +302,36 @@ def test_gemv_workspace_reset(ops):
     assert torch.equal(ops.gemv_forward(*args, ring=(2, 8, 4, 2)).view(torch.int16), want.view(torch.int16))
 
 
+def test_read_probes_do_read(ops):
+    """The floor probes must move their bytes (a reader whose result nothing observes compiles to an empty kernel): over
+    copies of a 235 MB weight that exceed the last-level cache, neither probe can beat 12 TB/s, and both take several
+    times an empty launch."""
+    from kairos_amd import _lib
+    lib = _lib.load()
+    N, K = 57344, 8192
+    nbytes = N * K // 2
+    qw = [torch.randint(-32768, 32767, (N // 4, K), dtype=torch.int16, device="cuda") for _ in range(3)]
+    st = ops._stream()
+
+    def timed(fn, n=12):
+        for i in range(3):
+            assert fn(i) == 0
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(n):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3 / n                   # seconds per launch
+
+    empty = timed(lambda i: lib.kmi_probe_empty(st))
+    plain = timed(lambda i: lib.kmi_probe_stream_read(qw[i % 3].data_ptr(), nbytes, st))
+    pattern = timed(lambda i: lib.kmi_probe_gemv_read(qw[i % 3].data_ptr(), N, K, 2, 8, st))
+    for t in (plain, pattern):
+        assert nbytes / t < 12e12 and t > 4 * empty, (empty, plain, pattern)
+
+
 # ------------------------------------------------------------------ MFMA GEMMs
 GEMM_M = [1, 7, 64, 65, 130, 300]
 
