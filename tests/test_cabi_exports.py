@@ -185,6 +185,19 @@ def test_tile_queries_survive_empty_products(lib):
     assert lib.kmi_gemm_w4a8_pick_tile(16, 4096, 0) == 128
 
 
+def test_w8a8_tile_rule_is_host_logic(lib):
+    """kmi_gemm_pick_tile (int8 operands): 256 x 192 tiles (selector 320) where N is a multiple of 384 and they make one
+    round or whole rounds while 256 x 256 tiles would leave a ragged one; 256 x 256 when those come in whole rounds; two
+    workgroups per CU on 256 x 128 tiles (192) where 256 x 256 tiles are too few and the rows too short to split."""
+    pick = lib.kmi_gemm_pick_tile
+    assert pick(2048, 6144, 4096) == 320          # 192 tiles of 256 x 256 against 256 of 256 x 192: one round
+    assert pick(4096, 6144, 4096) == 320          # 384 against 512: two whole rounds instead of 1.5
+    assert pick(8192, 6144, 4096) == 256          # 768 tiles of 256 x 256 are three whole rounds already
+    assert pick(4096, 28672, 4096) == 256 and pick(4096, 4096, 14336) == 256
+    assert pick(2048, 4096, 14336) == 192
+    assert pick(64, 4096, 4096) == 64
+
+
 def test_conversion_cache_handle_keeps_the_bound(lib):
     """The C-side bookkeeping of the bounded conversion buffer: hits only for the very copy the buffer holds, a request
     beyond the buffer is refused, invalidation forgets."""
