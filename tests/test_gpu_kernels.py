@@ -383,6 +383,31 @@ def test_gemm_w8a8_path(ops, M, tile):
     assert_same_bits(host(out), ref)
 
 
+@pytest.mark.parametrize("tile", [0, 64, 128, 256])
+def test_gemm_w8a8_subnormal_token_scales(ops, tile):
+    """Tokens whose largest value is below 127 * 2^-14 have a per-token scale that is subnormal in fp16 (down to the
+    smallest one, 2^-24), and the epilogue forms scale products on the matrix pipe: they must come out as exactly as the
+    oracle's fp32 products do (a pipe that flushed subnormal fp16 inputs would return zeros for these rows)."""
+    M, N, K = 70, 256, 512
+    p = prep(N, K)
+    x = O.synth_acts(M, K, seed=77).astype(np.float32)
+    x[::3] *= 1e-4                                            # scales around 3e-6
+    x[1::7] *= 1e-6                                           # scales of one or two units of 2^-24
+    x = x.astype(np.float16)
+    a8_np, sx_np = O.quant_act_i8(x)
+    sub = (sx_np.astype(np.float32) < 2.0 ** -14) & (sx_np.astype(np.float32) > 0)
+    assert sub.sum() >= 20                                    # the case is what it says
+    _, ref = O.gemm_w8a8(a8_np, p["w8"], p["scales_1"], sx_np)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.force_gemm_tile(tile)
+    try:
+        ops.w8a8_gemm_forward(dev(a8_np), dev(p["w8"]), dev(p["scales_1"]), dev(sx_np), out)
+    finally:
+        ops.force_gemm_tile(0)
+    assert_same_bits(host(out), ref)
+    assert np.abs(host(out)[sub].astype(np.float32)).max() > 0
+
+
 @pytest.mark.parametrize("tile", [0, 128, 130, 192, 256, 512])  # 130: the 128 x 128 tile with two wave quartets; 512: 512 x 128
 @pytest.mark.parametrize("M", GEMM_M)
 def test_gemm_w4a8_bit_exact(ops, M, tile):
