@@ -269,7 +269,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& p, acc_t (&acc)[FM
         half_t* outp = static_cast<half_t*>(p.out);
         const bool wide = (N & 7) == 0;                  // 16-byte row segments stay aligned
         // a tile inside the matrix: stores relative to the tile's origin, 32-bit offsets (256 rows of N fp16)
-        const bool inside = wide && m0 + BM <= M && n0 + BN <= N && (64 % CPR) == 0;
+        const bool inside = wide && m0 + BM <= M && n0 + BN <= N && (64 % CPR) == 0 && (long)N * BM * 2 < (1L << 32);
         const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(outp + ((long)m0 * N + n0), 0, -1, 0x00020000);
         const uint32_t ovoff = (uint32_t)(((wm * (BM / 2) + lane / CPR) * N + wn * WN + (lane % CPR) * 8) * 2);
         // Factor tiles, two in flight: tile t+1 is issued before tile t is converted.  Written as asm with a VGPR
