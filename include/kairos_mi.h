@@ -234,6 +234,23 @@ int kmi_gemm_w4a8_acc_i32(void* acc_i32, const void* a8, const void* qweight, co
                           void* workspace, size_t workspace_bytes, void* stream);
 int kmi_gemm_w4a8_pick_tile(int M, int N, int K);
 
+/* W4A8 with INTEGER per-group factors, the arithmetic of the version-2 candidate itself (kairos/dynamic_linear_v2.py:161-179
+ * -> qgemm_w4a8_per_group.gemm_forward_cuda, thirdparty/Qserve/qserve_kernels/csrc/qgemm/w4a8_per_group/gemm_cuda.cu:299-329,
+ * 620-627), read from the resident packed int4 weight (no trans_layout_c16_to_c8_awq call in front):
+ *   W8[n,k] = (int8)((q[n,k] * s2_scales[k/G,n] + s2_zeros[k/G,n]) mod 256),  acc = a8 . W8^T,
+ *   out = fp16(float(acc) * (float(wscales[n]) * float(ascales[m]))) (+bias).
+ * s2_scales / s2_zeros: int8 [K/G, N] in plain column order (the reference stores them shuffled inside blocks of 32 columns
+ * for its tensor-core fragments, thirdparty/Qserve/w4a8_linear.py:215-262); s2_scales is read as an unsigned byte, s2_zeros
+ * is the negated zero point times the scale as a two's-complement byte.  Every weight byte wraps on its own; the CUDA kernel
+ * multiplies four packed bytes at once and agrees as long as 15 * scale < 256, which its quantiser guarantees.
+ * Same tiles, workspace and selectors as kmi_gemm_w4a8. */
+int kmi_gemm_w4a8_int(void* out_f16, const void* a8, const void* qweight, const void* s2_scales_i8, const void* s2_zeros_i8,
+                      const void* wscales_f16, const void* ascales_f16, const void* bias, int M, int N, int K, int G,
+                      void* workspace, size_t workspace_bytes, void* stream);
+int kmi_gemm_w4a8_int_acc_i32(void* acc_i32, const void* a8, const void* qweight, const void* s2_scales_i8,
+                              const void* s2_zeros_i8, int M, int N, int K, int G,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
 /* FP16: out = x . w16^T (+bias), fp32 accumulation.  Replaces `input @ tmp_weight.T`
  * (kairos/dynamic_linear.py:163). */
 int kmi_gemm_f16(void* out_f16, const void* x_f16, const void* w16, const void* bias,

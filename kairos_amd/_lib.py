@@ -44,6 +44,8 @@ SIGNATURES = {
     "kmi_gemm_w4a8": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w4a8_acc_i32": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w4a8_pick_tile": [_I, _I, _I],
+    "kmi_gemm_w4a8_int": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
+    "kmi_gemm_w4a8_int_acc_i32": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_f16": [_P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_w8a8_tiled": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],
     "kmi_gemm_f16_tiled": [_P, _P, _P, _P, _I, _I, _I, _P, _Z, _P],

@@ -44,6 +44,18 @@ __device__ __forceinline__ uint32_t w4a8_table_word_of(h2_t q01, h2_t q23, half_
     return pack_i8x4(pk_fma(q01, s2, z2), pk_fma(q23, s2, z2));
 }
 
+// Integer factors (the form a per-group integer dequantiser uses): table byte q = (q * scale + zero) modulo 256 read as
+// int8, `scale` an unsigned byte, `zero` the pre-multiplied (negated) zero point as a byte.  `wbase` holds the four nibble
+// values of the word, one per byte.  The products are taken per byte pair so that no carry crosses a byte, whatever the
+// scale; the add wraps per byte.
+__device__ __forceinline__ uint32_t w4a8_table_word_int(uint32_t wbase, uint32_t scale, uint32_t zero) {
+    const uint32_t even = ((wbase & 0x00FF00FFu) * (scale & 0xFFu)) & 0x00FF00FFu;
+    const uint32_t odd = (((wbase >> 8) & 0x00FF00FFu) * (scale & 0xFFu)) & 0x00FF00FFu;
+    const uint32_t prod = even | (odd << 8);
+    const uint32_t z4 = zero * 0x01010101u;
+    return ((prod & 0x7F7F7F7Fu) + (z4 & 0x7F7F7F7Fu)) ^ ((prod ^ z4) & 0x80808080u);
+}
+
 // Four nibbles (`idx3`: their low three bits, one per byte; `sel_hi`: 0x03020100 + 4 * bit 3, one per byte) -> four
 // table bytes.
 __device__ __forceinline__ uint32_t w4a8_lookup(const uint32_t (&L)[4], uint32_t idx3, uint32_t sel_hi) {
@@ -98,7 +110,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 // MFMAs -- queues on that wave's own issue port, which the MFMAs cannot cover, and a 64-lane load holds the port far
 // longer than a vector instruction; with the roles apart the decoding wave never waits behind a load, and the second
 // wave of the SIMD issues its MFMAs, fragment reads and loads into the gaps of the first.
-template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
+//
+// INTF: the per-group factors are integers -- `p.scales` / `p.szeros` point to int8 tables [K/128][N] (scale byte and
+// pre-multiplied negated zero byte) and the table of a group is (q * scale + zero) modulo 256; everything else is the same.
+template <int KIND, int BM, int BN, int KH = 1, int MW = 1, bool INTF = false>
 __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     static_assert(KIND == KIND_W8A8 || KIND == KIND_W8A8_ACC, "int8 accumulation");
@@ -159,7 +174,8 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     int ncol = n0 + brow;
     ncol = ncol < N ? ncol : N - 1;                          // ragged last tile: clamp loads, stores are masked
     const uint32_t voff_b = (uint32_t)((long)(ncol >> 2) * K * 2 + (ncol & 3) * 32 + (CPT == 2 ? 0 : (tid & 1) * 16));
-    const uint32_t voff_s = (uint32_t)ncol * 2u;
+    const uint32_t voff_s = (uint32_t)ncol * (INTF ? 1u : 2u);
+    constexpr uint32_t SZB = INTF ? 1u : 2u;                // bytes per table entry
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.a), 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.b), 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(p.scales), 0, -1, 0x00020000);
@@ -174,6 +190,10 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     uint32_t L[4];
 
     auto clamp_stage = [&](int u) { return t0 + (u < T ? u : T - 1); };   // past the end: harmless reloads
+    auto load_factor = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t so) -> unsigned short {
+        if constexpr (INTF) return (unsigned short)__builtin_amdgcn_raw_buffer_load_b8(rsrc, voff_s, so, 0);
+        else return (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, voff_s, so, 0);
+    };
     auto issue_raw = [&](int u, auto sp, auto gp) {
         const uint32_t sb = (uint32_t)clamp_stage(u) * 128u;
 #pragma unroll
@@ -182,9 +202,9 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
                 __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b + 16u * j, sb, 0));
     };
     auto issue_sz = [&](int u, auto gp) {                    // scale and scaled zero of the group of (even) stage u
-        const uint32_t so = (uint32_t)(clamp_stage(u) >> 1) * (uint32_t)N * 2u;
-        sraw[decltype(gp)::value] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_s, voff_s, so, 0);
-        zraw[decltype(gp)::value] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_z, voff_s, so, 0);
+        const uint32_t so = (uint32_t)(clamp_stage(u) >> 1) * (uint32_t)N * SZB;
+        sraw[decltype(gp)::value] = load_factor(rsrc_s, so);
+        zraw[decltype(gp)::value] = load_factor(rsrc_z, so);
     };
     // ---- the decode work of one iteration as a list of small items (compile-time index), placed one by one between
     // the MFMAs.  Items of an iteration that decodes stage u (stage parity SP, group parity GN of u):
@@ -198,9 +218,12 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
     // values 8*hsel .. 8*hsel+7 and gets the other half from its neighbour with a lane swap inside the quad.
     h2_t tq[4];                                              // the eight nibble values of this thread's half, as fp16 pairs
     uint32_t town[2], tnbr[2];
+    uint32_t wb[2];                                          // INTF: the same eight values, one per byte
     if constexpr (CPT == 1) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) tq[i] = h2_t{(half_t)(float)(8 * hsel + 2 * i), (half_t)(float)(8 * hsel + 2 * i + 1)};
+        wb[0] = 0x03020100u + 0x08080808u * (uint32_t)hsel;
+        wb[1] = 0x07060504u + 0x08080808u * (uint32_t)hsel;
     }
     auto work_item = [&](auto sp, auto gn, auto with_table, auto item, int slot) {
         constexpr int SPv = decltype(sp)::value, GNv = decltype(gn)::value, IT = decltype(item)::value;
@@ -208,9 +231,11 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
         if constexpr (IT < NT) {
             const half_t sc = __builtin_bit_cast(half_t, sraw[GNv]), zc = __builtin_bit_cast(half_t, zraw[GNv]);
             if constexpr (CPT == 2) {
-                L[IT] = w4a8_table_word<IT>(sc, zc);
+                if constexpr (INTF) L[IT] = w4a8_table_word_int(0x03020100u + 0x04040404u * IT, sraw[GNv], zraw[GNv]);
+                else L[IT] = w4a8_table_word<IT>(sc, zc);
             } else if constexpr (IT < 2) {
-                town[IT] = w4a8_table_word_of(tq[2 * IT], tq[2 * IT + 1], sc, zc);
+                if constexpr (INTF) town[IT] = w4a8_table_word_int(wb[IT], sraw[GNv], zraw[GNv]);
+                else town[IT] = w4a8_table_word_of(tq[2 * IT], tq[2 * IT + 1], sc, zc);
             } else if constexpr (IT == 2) {                  // quad_perm [1, 0, 3, 2]: the other thread of the row
                 tnbr[0] = (uint32_t)__builtin_amdgcn_mov_dpp((int)town[0], 0xB1, 0xF, 0xF, true);
                 tnbr[1] = (uint32_t)__builtin_amdgcn_mov_dpp((int)town[1], 0xB1, 0xF, 0xF, true);
@@ -325,7 +350,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
         wait_vmcnt<NLA1 + NLA0 + CPE + (SP == 1 ? SZ : 0)>();
         const uint32_t sa3 = (uint32_t)clamp_stage(t + 3) * 64u, sa4 = (uint32_t)clamp_stage(t + 4) * 64u;
         const uint32_t sb4 = (uint32_t)clamp_stage(t + 4) * 128u;
-        const uint32_t so4 = (uint32_t)(clamp_stage(t + 4) >> 1) * (uint32_t)N * 2u;
+        const uint32_t so4 = (uint32_t)(clamp_stage(t + 4) >> 1) * (uint32_t)N * SZB;
         static_for<0, NSLOTS>([&](auto q_) {
             constexpr int Q = decltype(q_)::value, BLK = Q / NMF, q = Q % NMF;
             if constexpr (Q == NMF)      // stage t+1 is complete for every wave and stage t is in registers
@@ -354,9 +379,9 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
                 } else if constexpr (l < NLA0 + CPE) {       // packed chunks of stage t+4
                     raw[SP][GP][l - NLA0] = __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b + 16u * (l - NLA0), sb4, 0));
                 } else if constexpr (l == NLA0 + CPE) {      // scale / scaled zero of the group stage t+4 opens
-                    sraw[GP] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_s, voff_s, so4, 0);
+                    sraw[GP] = load_factor(rsrc_s, so4);
                 } else {
-                    zraw[GP] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc_z, voff_s, so4, 0);
+                    zraw[GP] = load_factor(rsrc_z, so4);
                 }
             });
             // the slot's MFMA
@@ -427,7 +452,7 @@ __global__ __launch_bounds__(256 * KH * MW) void gemm_w4a8_kernel(GemmArgs p) {
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-template <int KIND, int BM, int BN, int KH = 1, int MW = 1>
+template <int KIND, bool INTF, int BM, int BN, int KH = 1, int MW = 1>
 static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t st, int n_begin = 0, int n_cols = -1) {
     GemmArgs a = a_in;
     a.group_m = kmi_forced_group_m();
@@ -435,7 +460,7 @@ static int launch_w4a8(const GemmArgs& a_in, const Workspace& ws_in, hipStream_t
     a.n_cols = n_cols < 0 ? a.N - n_begin : n_cols;
     const Workspace ws = (a.n_begin == 0 && a.n_cols == a.N) ? ws_in : Workspace{nullptr, 0};   // column ranges: no split over K
     constexpr size_t lds = (size_t)KH * 4 * (BM + BN) * 64;
-    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN, KH, MW>;
+    void (*fn)(GemmArgs) = gemm_w4a8_kernel<KIND, BM, BN, KH, MW, INTF>;
     static thread_local bool raised = false;                 // per instantiation, per thread
     if (lds > 64 * 1024 && !raised) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -560,7 +585,7 @@ static int w4a8_tile(int M, int N, int K) {
 }
 extern "C" int kmi_gemm_w4a8_pick_tile(int M, int N, int K) { return w4a8_tile(M, N, K); }
 
-template <int KIND>
+template <int KIND, bool INTF = false>
 static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace, size_t workspace_bytes, void* stream) {
     if (G != 128) return kmi_set_error(KMI_E_GROUP, "%s: group size %d unsupported (128 only)", fn, G);
     if (!a.scales || !a.szeros) return kmi_set_error(KMI_E_NULL, "%s: NULL scale table", fn);
@@ -575,17 +600,17 @@ static int w4a8_entry(const char* fn, GemmArgs& a, int G, const void* workspace,
     const int tile = w4a8_tile(a.M, a.N, a.K);
     if (tile == 640) {
         const int head = w4a8_head_cols_512(a.M, a.N) * 128;
-        rc = launch_w4a8<KIND, 512, 128, 1, 2>(a, ws, st, 0, head);
-        if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
+        rc = launch_w4a8<KIND, INTF, 512, 128, 1, 2>(a, ws, st, 0, head);
+        if (rc == KMI_OK) rc = launch_w4a8<KIND, INTF, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
     } else if (tile == 448) {
         const int head = w4a8_head_cols(a.M, a.N) * 256;
-        rc = launch_w4a8<KIND, 256, 256>(a, ws, st, 0, head);
-        if (rc == KMI_OK) rc = launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
+        rc = launch_w4a8<KIND, INTF, 256, 256>(a, ws, st, 0, head);
+        if (rc == KMI_OK) rc = launch_w4a8<KIND, INTF, 256, 128, 1, 2>(a, ws, st, head, a.N - head);
     } else {
-        rc = tile == 256 ? launch_w4a8<KIND, 256, 256>(a, ws, st)
-           : tile == 192 ? launch_w4a8<KIND, 256, 128, 1, 2>(a, ws, st)
-           : tile == 130 ? launch_w4a8<KIND, 128, 128, 2>(a, ws, st)
-           : tile == 512 ? launch_w4a8<KIND, 512, 128, 1, 2>(a, ws, st) : launch_w4a8<KIND, 128, 128>(a, ws, st);
+        rc = tile == 256 ? launch_w4a8<KIND, INTF, 256, 256>(a, ws, st)
+           : tile == 192 ? launch_w4a8<KIND, INTF, 256, 128, 1, 2>(a, ws, st)
+           : tile == 130 ? launch_w4a8<KIND, INTF, 128, 128, 2>(a, ws, st)
+           : tile == 512 ? launch_w4a8<KIND, INTF, 512, 128, 1, 2>(a, ws, st) : launch_w4a8<KIND, INTF, 128, 128>(a, ws, st);
     }
     if (rc != KMI_OK) return rc;
     return kmi_check_launch(fn);
@@ -605,4 +630,22 @@ extern "C" int kmi_gemm_w4a8_acc_i32(void* acc, const void* a8, const void* qwei
     GemmArgs a{acc, a8, qweight, (const half_t*)scales_to8, (const half_t*)szeros_to8, nullptr, nullptr, nullptr, M, N, K,
                nullptr, 1, 0, N};
     return w4a8_entry<KIND_W8A8_ACC>("kmi_gemm_w4a8_acc_i32", a, G, workspace, workspace_bytes, stream);
+}
+
+// The same product with integer per-group factors: int8 tables [K/128][N] in plain column order, weight byte =
+// (q * scale + zero) modulo 256 read as int8.
+extern "C" int kmi_gemm_w4a8_int(void* out, const void* a8, const void* qweight, const void* s2_scales_i8, const void* s2_zeros_i8,
+                                 const void* wscales, const void* ascales, const void* bias, int M, int N, int K, int G,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    GemmArgs a{out, a8, qweight, (const half_t*)s2_scales_i8, (const half_t*)s2_zeros_i8, (const half_t*)wscales,
+               (const half_t*)ascales, (const half_t*)bias, M, N, K, nullptr, 1, 0, N};
+    return w4a8_entry<KIND_W8A8, true>("kmi_gemm_w4a8_int", a, G, workspace, workspace_bytes, stream);
+}
+
+extern "C" int kmi_gemm_w4a8_int_acc_i32(void* acc, const void* a8, const void* qweight, const void* s2_scales_i8,
+                                         const void* s2_zeros_i8, int M, int N, int K, int G, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    GemmArgs a{acc, a8, qweight, (const half_t*)s2_scales_i8, (const half_t*)s2_zeros_i8, nullptr, nullptr, nullptr, M, N, K,
+               nullptr, 1, 0, N};
+    return w4a8_entry<KIND_W8A8_ACC, true>("kmi_gemm_w4a8_int_acc_i32", a, G, workspace, workspace_bytes, stream);
 }

@@ -421,6 +421,45 @@ def w4a8_gemm_acc_i32(in_feats, qweight, scales_to8, scaled_zeros_to8):
     return acc
 
 
+def _need_int_tables(name, s2_scales, s2_zeros, N, K):
+    for t, what in ((s2_scales, "s2_scales"), (s2_zeros, "s2_zeros")):
+        _need(t, torch.int8, what)
+        if t.dim() != 2 or t.shape[0] < K // GROUP_SIZE or t.shape[1] != N:
+            raise ValueError(f"{name}: {what} must be int8 [K/{GROUP_SIZE}, N] = [{K // GROUP_SIZE}, {N}], got {tuple(t.shape)}")
+
+
+def w4a8_int_gemm_forward(in_feats, qweight, s2_scales, s2_zeros, wscales, ascales, out_feats, bias=None):
+    """out_feats fp16 [M, N] <- int8 [M, K] x packed int4 [N/4, K] with integer per-group factors: the arithmetic of
+    omniserve_backend.qgemm_w4a8_per_group.gemm_forward_cuda as the version-2 layer calls it
+    (kairos/dynamic_linear_v2.py:161-179), on the resident weight (no re-pack) and with the int8 tables [K/128, N] in
+    plain column order: weight byte = (q * s2_scales + s2_zeros) mod 256."""
+    _need(in_feats, torch.int8, "in_feats"); _need(qweight, torch.int16, "qweight"); _need(out_feats, torch.float16, "out_feats")
+    M, K = in_feats.shape
+    N = qweight.shape[0] * 4
+    if qweight.shape[1] != K or out_feats.shape[-1] != N:
+        raise ValueError(f"w4a8_int_gemm_forward: activations [{M}, {K}], weight [{N}, {qweight.shape[1]}], output {tuple(out_feats.shape)}")
+    _need_int_tables("w4a8_int_gemm_forward", s2_scales, s2_zeros, N, K)
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
+    _call("gemm_w4a8_int", M, N, K, _lib.load().kmi_gemm_w4a8_int, out_feats.data_ptr(), in_feats.data_ptr(), qweight.data_ptr(),
+          s2_scales.data_ptr(), s2_zeros.data_ptr(), wscales.data_ptr(), ascales.data_ptr(), _ptr(bias), M, N, K,
+          GROUP_SIZE, ws.data_ptr(), ws.numel(), st)
+
+
+def w4a8_int_gemm_acc_i32(in_feats, qweight, s2_scales, s2_zeros):
+    """Raw int32 accumulators [M, N] of the integer-factor W4A8 product."""
+    _need(in_feats, torch.int8, "in_feats"); _need(qweight, torch.int16, "qweight")
+    M, K = in_feats.shape
+    N = qweight.shape[0] * 4
+    _need_int_tables("w4a8_int_gemm_acc_i32", s2_scales, s2_zeros, N, K)
+    acc = torch.empty((M, N), dtype=torch.int32, device=in_feats.device)
+    st = _stream()
+    ws = workspace_for(in_feats.device, st)
+    _lib.check(_lib.load().kmi_gemm_w4a8_int_acc_i32(acc.data_ptr(), in_feats.data_ptr(), qweight.data_ptr(), s2_scales.data_ptr(),
+                                                     s2_zeros.data_ptr(), M, N, K, GROUP_SIZE, ws.data_ptr(), ws.numel(), st))
+    return acc
+
+
 def w8a8_gemm_acc_i32(in_feats, kernel, N):
     """Raw int32 accumulators [M, N] of the W8A8 product."""
     _need(in_feats, torch.int8, "in_feats"); _need(kernel, torch.int8, "kernel")

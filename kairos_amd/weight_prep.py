@@ -4,7 +4,10 @@ ops on whatever device the weight lives on.
 
 Mirrors kairos/quantization.py:112-141 (quantize_tensor_int8), kairos/dynamic_linear_v2.py:15-41
 (kairos_quantize_tensor_int4) and thirdparty/AWQ/awq_method.py:5-75 (pack_int_awq,
-calculate_zeros_width, trans_qfactor_layout_awq): same names, arguments and results.
+calculate_zeros_width, trans_qfactor_layout_awq): same names, arguments and results.  The second
+quantiser whose integer factors the version-2 `w4a8_qserve` candidate multiplies with
+(thirdparty/Qserve/quantization.py:4-36, tables of thirdparty/Qserve/w4a8_linear.py:215-262) is
+here as well: qserve_quantize_tensor_int8 / _int4 and qserve_factor_tables.
 """
 import torch
 
@@ -127,3 +130,53 @@ def prepare_linear_weight(weight, group_size=128):
     return {"qweight": pack_int_awq(q4), "scales": scales, "scaled_zeros": scaled_zeros,
             "scales_to8": scales_to8, "scaled_zeros_to8": scaled_zeros_to8,
             "scales_1": scale_1.reshape(-1).contiguous()}
+
+
+@torch.no_grad()
+def qserve_quantize_tensor_int8(x, return_dtype=torch.float16):
+    """Per-row symmetric int8 inside the protective range +-119 (thirdparty/Qserve/quantization.py:4-15)."""
+    shape = x.shape
+    rows = x.reshape(-1, shape[-1]).to(torch.float32)
+    step = rows.abs().amax(dim=1, keepdim=True).clamp(min=1e-7) / 119
+    q = torch.round(rows / step).to(torch.int8)
+    if torch.isnan(rows).any():
+        raise ValueError("NaN while quantising to int8")
+    return q.reshape(shape), {"scale": step.to(return_dtype)}
+
+
+@torch.no_grad()
+def qserve_quantize_tensor_int4(x, group_size=-1):
+    """int8 -> uint4 per group with whole-number scale and zero point (thirdparty/Qserve/quantization.py:17-36):
+    scale = round(range / 15) (0 becomes 1), zero = round(-min / scale), q = clamp(round(x / scale + zero), 0, 15)."""
+    shape = x.shape
+    if group_size < 0:
+        g = x.reshape(-1, shape[-1])
+    else:
+        if shape[-1] % group_size:
+            raise ValueError(f"last dimension {shape[-1]} is not a multiple of group_size {group_size}")
+        g = x.reshape(-1, group_size)
+    g = g.to(torch.float32)
+    lo = g.amin(dim=1, keepdim=True)
+    step = torch.round((g.amax(dim=1, keepdim=True) - lo).clamp(min=1e-7) / 15)
+    step[step == 0] = 1
+    zero = torch.round(-(lo / step))
+    q = torch.clamp(torch.round(g / step + zero), 0, 15)
+    return q.reshape(shape).to(torch.int8), {"scale": step.to(torch.int8), "zero_pt": zero.to(torch.int8),
+                                             "group_size": group_size}
+
+
+@torch.no_grad()
+def qserve_factor_tables(weight, group_size=128):
+    """The operands that W4A8Linear.from_module derives beside its own nibbles (thirdparty/Qserve/w4a8_linear.py:182-262)
+    and that the version-2 layer hands to the W4A8 GEMM with the RESIDENT nibbles (kairos/dynamic_linear_v2.py:103,
+    161-179): s1_scales fp16 [N], s2_scales int8 [K/G, N], s2_zeros int8 [K/G, N] = -(zero * scale) as a
+    two's-complement byte.  Plain column order: the shuffle inside blocks of 32 columns that the reference applies is
+    the fragment order of its CUDA kernel and has no meaning for the MFMA kernel that reads these tables."""
+    w = weight.detach().to(torch.float16).cpu()
+    N, K = w.shape
+    w8, cfg1 = qserve_quantize_tensor_int8(w)
+    _, cfg2 = qserve_quantize_tensor_int4(w8, group_size=group_size)
+    s2 = cfg2["scale"].reshape(N, K // group_size).t().contiguous()
+    z2 = cfg2["zero_pt"].reshape(N, K // group_size).t().contiguous()
+    zs = (-(z2.to(torch.int32) * s2.to(torch.int32))).to(torch.int8)          # wraps like the reference's int8 store
+    return {"s1_scales": cfg1["scale"].reshape(N).contiguous(), "s2_scales": s2, "s2_zeros": zs}

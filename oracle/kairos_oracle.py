@@ -25,10 +25,19 @@ Pinning status (what, other than this file agreeing with itself, fixes each func
                                   accumulated matmul, tolerance 1e-2 max-abs-rel.
   gemm_w8a16                      parity unpinned: the reference declares the id but has no
                                   implementation (kairos/dynamic_linear.py:8-9).
-  switched_forward, id 7          parity unpinned by the reference: its `w4a8_qserve` candidate calls an un-vendored
-                                  third-party GEMM with a quantiser of its own (kairos/dynamic_linear_v2.py:161-179).
-                                  The build's W4A8 lane is DEFINED as the W8A8 lane's product (same int8 weight,
-                                  decoded inside the GEMM), so its oracle is the pinned W8A8 chain, bit for bit.
+  switched_forward, id 7          the build's default W4A8 lane is DEFINED as the W8A8 lane's product (same int8
+                                  weight, decoded inside the GEMM), so its oracle is the pinned W8A8 chain, bit for
+                                  bit.  The reference's own `w4a8_qserve` candidate (kairos/dynamic_linear_v2.py:
+                                  161-179) feeds the resident nibbles to a CUDA GEMM with integer per-group factors
+                                  of a second quantiser; that arithmetic is restated below:
+  qserve_quantize_int8 / _int4    closed forms of thirdparty/Qserve/quantization.py:4-36; hand cases, the protective
+                                  range (|w8| <= 119 keeps q*s - z*s inside int8, so the byte-wise wrap never
+                                  fires), reconstruction error <= s/2 per element.
+  dequant_w4a8_int / gemm_w4a8_   the kernel's register arithmetic (thirdparty/Qserve/qserve_kernels/csrc/qgemm/
+  int                             w4a8_per_group/gemm_cuda.cu:299-329: byte-wise q*s + z') and its epilogue
+                                  (:620-627); pinned by textbook (q - zero) * scale on the quantiser's own output,
+                                  by wrap-around hand cases, and by the exact integer matmul.  No output of the
+                                  CUDA kernel exists in the reference to compare with (it cannot be built here).
   pack_int_w4a8 / trans_layout_   the reference states the layout twice (test/test_trans_layout.py:8-14 in one
   c16_to_c8                       permutation, thirdparty/Qserve/w4a8_linear.py:187-205 in two) and its own test
                                   demands trans(pack_awq(A)) == pack_w4a8(A) bit for bit (test_trans_layout.py:46-52);
@@ -316,6 +325,62 @@ def dequant_to_i8(qweight, scales_to8, scaled_zeros_to8, group_size=GROUP):
     f = dequant_to_f16(qweight, scales_to8, scaled_zeros_to8, group_size).astype(np.float32)
     f = np.where(np.isnan(f), np.float32(0), f)
     return np.clip(np.trunc(f), -128, 127).astype(np.int8)
+
+
+# ----------------------------------------------------------------------------------------------
+# The reference's own id-7 operands: integer per-group factors on top of a per-channel int8 level
+# ----------------------------------------------------------------------------------------------
+def qserve_quantize_int8(w):
+    """thirdparty/Qserve/quantization.py:4-15: per-row symmetric int8 with the protective range 119.
+    fp [N, K] -> (int8 [N, K], scale fp16 [N, 1]); the division uses the fp32 scale, the fp16 one is what is stored."""
+    x = np.asarray(w).astype(np.float32)
+    mx = np.maximum(np.abs(x).max(axis=1, keepdims=True), np.float32(1e-7))
+    scale = (mx / np.float32(119)).astype(np.float32)
+    return np.rint(x / scale).astype(np.int8), scale.astype(np.float16)
+
+
+def qserve_quantize_int4(w8, group_size=GROUP):
+    """thirdparty/Qserve/quantization.py:17-36: int8 -> uint4 per group with WHOLE-NUMBER scale and zero point.
+    scale = round((max - min).clamp(1e-7) / 15), 0 -> 1; zero = round(-min / scale); q = clamp(round(x / scale + zero)).
+    -> (uint4-in-int8 [N, K], scale int8 [N*K/G, 1], zero int8 [N*K/G, 1])"""
+    w8 = np.asarray(w8)
+    shape = w8.shape
+    assert shape[-1] % group_size == 0
+    x = w8.reshape(-1, group_size).astype(np.float32)
+    mx = x.max(axis=1, keepdims=True)
+    mn = x.min(axis=1, keepdims=True)
+    scale = np.rint(np.maximum(mx - mn, np.float32(1e-7)) / np.float32(15))
+    scale[scale == 0] = 1
+    zero = np.rint(-(mn / scale))
+    q = np.clip(np.rint(x / scale + zero), 0, 15)
+    return q.reshape(shape).astype(np.int8), scale.astype(np.int8), zero.astype(np.int8)
+
+
+def qserve_tables(scale_i, zero_i, N, group_size=GROUP):
+    """thirdparty/Qserve/w4a8_linear.py:215-262 without the 32-column shuffle the CUDA fragments want: per-group tables
+    [K/G, N] in plain column order, s2_scales = scale, s2_zeros = int8(-zero * scale) (two's complement, wrapping)."""
+    s = np.asarray(scale_i).reshape(N, -1).T.astype(np.int32)
+    z = np.asarray(zero_i).reshape(N, -1).T.astype(np.int32)
+    return s.astype(np.int8), ((-z * s) & 0xFF).astype(np.uint8).view(np.int8)
+
+
+def dequant_w4a8_int(qweight, s2_scales, s2_zeros, group_size=GROUP):
+    """gemm_cuda.cu:299-329 of the per-group W4A8 kernel: every weight byte is (q * scale + zeros') modulo 256, read
+    as int8 -- a packed 32-bit multiply by the scale byte (no carry between bytes while 15 * scale < 256, which the
+    quantiser guarantees) and a byte-wise wrapping add of the pre-multiplied zero.  Here each byte is taken modulo
+    256 on its own, for any scale byte (read as unsigned, as the kernel's mask does)."""
+    N, K = qweight.shape[0] * 4, qweight.shape[1]
+    ng = K // group_size
+    q = unpack_int_awq(qweight).reshape(N, ng, group_size).astype(np.int32)
+    s = (np.asarray(s2_scales)[:ng].astype(np.int32) & 0xFF).T[:, :, None]
+    z = (np.asarray(s2_zeros)[:ng].astype(np.int32) & 0xFF).T[:, :, None]
+    return ((q * s + z) & 0xFF).astype(np.uint8).view(np.int8).reshape(N, K)
+
+
+def gemm_w4a8_int(a8, qweight, s2_scales, s2_zeros, wscales, ascales, group_size=GROUP):
+    """The reference's id-7 product (kairos/dynamic_linear_v2.py:161-179; epilogue gemm_cuda.cu:620-627, the same
+    order as the W8A8 kernel's): int32 accumulators and fp16 output."""
+    return gemm_w8a8(a8, dequant_w4a8_int(qweight, s2_scales, s2_zeros, group_size), wscales, ascales)
 
 
 # ----------------------------------------------------------------------------------------------

@@ -546,6 +546,84 @@ def test_gemm_w4a8_random_tables_and_splits(ops, tile, splits):
     assert torch.equal(acc, again) and torch.equal(acc, ops.w8a8_gemm_acc_i32(a8, w8, N))
 
 
+def _int_factor_case(N, K, seed):
+    """A weight through both quantisers of the version-2 layer: the resident nibbles (this layer's own) and the integer
+    factors of the second quantiser (what its id 7 multiplies them with)."""
+    w = O.synth_weights(N, K, seed)
+    p = O.prepare_weights(w)
+    w8, s1 = O.qserve_quantize_int8(w)
+    _, si, zi = O.qserve_quantize_int4(w8)
+    S, Z = O.qserve_tables(si, zi, N)
+    return p["qweight"], S, Z, s1.reshape(-1)
+
+
+@pytest.mark.parametrize("tile", [0, 128, 130, 192, 256, 512])
+@pytest.mark.parametrize("M", [1, 33, 300])
+def test_gemm_w4a8_int_factors_bit_exact(ops, M, tile):
+    """W4A8 with integer per-group factors (the arithmetic of the version-2 candidate's own GEMM,
+    thirdparty/Qserve/qserve_kernels/csrc/qgemm/w4a8_per_group/gemm_cuda.cu:299-329, 620-627): int32 accumulators and
+    fp16 outputs, with and without a bias, against the oracle bit for bit; N = 384 leaves every tile ragged."""
+    N, K = 384, 1024
+    qw_np, S, Z, s1 = _int_factor_case(N, K, seed=tile + 1)
+    x = O.synth_acts(M, K, seed=900 + M)
+    a8, sx = O.quant_act_i8(x)
+    acc_ref, out_ref = O.gemm_w4a8_int(a8, qw_np, S, Z, s1, sx)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float16)
+    out_b_ref = (out_ref.astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    qw, s2, z2 = dev(qw_np), dev(S), dev(Z)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    out_b = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(1)
+    try:
+        acc = ops.w4a8_int_gemm_acc_i32(dev(a8), qw, s2, z2)
+        ops.w4a8_int_gemm_forward(dev(a8), qw, s2, z2, dev(s1), dev(sx), out)
+        ops.w4a8_int_gemm_forward(dev(a8), qw, s2, z2, dev(s1), dev(sx), out_b, bias=dev(bias))
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert_same_bits(host(acc), acc_ref)
+    assert_same_bits(host(out), out_ref)
+    assert_same_bits(host(out_b), out_b_ref)
+
+
+@pytest.mark.parametrize("tile,splits", [(128, 1), (256, 2), (192, 1), (192, 4), (130, 2), (512, 1), (512, 2), (0, 0)])
+def test_gemm_w4a8_int_factors_any_bytes_and_splits(ops, tile, splits):
+    """Arbitrary nibbles and arbitrary factor bytes (scales up to 255, negative bytes): every weight byte wraps modulo
+    256 on its own, as the oracle's does; full-range activations, K split over workgroups."""
+    rng = np.random.default_rng(tile + splits)
+    N, K, M = 512, 2048, 200
+    qw_np = rng.integers(-32768, 32768, size=(N // 4, K), dtype=np.int16)
+    S = rng.integers(-128, 128, size=(K // 128, N), dtype=np.int8)
+    Z = rng.integers(-128, 128, size=(K // 128, N), dtype=np.int8)
+    a8_np = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w8_ref = O.dequant_w4a8_int(qw_np, S, Z)
+    assert w8_ref.min() == -128 and w8_ref.max() == 127
+    ops.force_gemm_tile(tile)
+    ops.force_gemm_splits(splits)
+    try:
+        acc = ops.w4a8_int_gemm_acc_i32(dev(a8_np), dev(qw_np), dev(S), dev(Z))
+        again = ops.w4a8_int_gemm_acc_i32(dev(a8_np), dev(qw_np), dev(S), dev(Z))
+    finally:
+        ops.force_gemm_tile(0)
+        ops.force_gemm_splits(0)
+    assert_same_bits(host(acc), O.gemm_i8_acc(a8_np, w8_ref))
+    assert torch.equal(acc, again)
+    assert torch.equal(acc, ops.w8a8_gemm_acc_i32(dev(a8_np), dev(w8_ref), N))
+
+
+def test_gemm_w4a8_int_factors_reject_wrong_tables(ops):
+    qw = torch.zeros((64, 256), dtype=torch.int16, device="cuda")
+    a8 = torch.zeros((4, 256), dtype=torch.int8, device="cuda")
+    good = torch.zeros((2, 256), dtype=torch.int8, device="cuda")
+    with pytest.raises(TypeError):
+        ops.w4a8_int_gemm_acc_i32(a8, qw, good.half(), good)
+    with pytest.raises(ValueError):
+        ops.w4a8_int_gemm_acc_i32(a8, qw, good[:1], good)
+    with pytest.raises(ValueError):
+        ops.w4a8_int_gemm_acc_i32(a8, qw, good, good[:, :128].contiguous())
+
+
 @pytest.mark.parametrize("K,N,wide", [(128, 7808, 256), (384, 7808, 256), (384, 7680, 320), (128, 7808, 320)])
 def test_gemm_256_tile_walking_several_tiles_per_workgroup(ops, K, N, wide):
     """More 256 x 256 tiles than compute units (9 x 31 = 279, ragged in M and N): the tiled-weight W8A8 and fp16 GEMMs

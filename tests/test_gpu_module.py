@@ -210,6 +210,48 @@ def test_graph_replay_matches_eager():
         DynamicLinear.prof = old
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_version2_layer_with_the_reference_w4a8_operands(gpu, bias, tmp_path):
+    """from_module(..., qserve_factors=True): id 7 multiplies the resident nibbles with the integer factors and the
+    per-channel scale of the second quantiser, as kairos/dynamic_linear_v2.py:103,161-179 does -- the oracle's
+    restatement of that GEMM bit for bit, the other lanes untouched, and the three extra tensors travel in the state dict."""
+    from kairos.dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear
+    N, K = 256, 1024
+    lin, w = make_linear(N, K, bias, seed=31)
+    plain = DynamicLinear.from_module(lin.cuda(), 'cuda')
+    dl = DynamicLinear.from_module(lin, 'cuda', qserve_factors=True)
+    w8, s1 = O.qserve_quantize_int8(w)
+    _, si, zi = O.qserve_quantize_int4(w8)
+    S, Z = O.qserve_tables(si, zi, N)
+    assert np.array_equal(dl.qserve_s2_scales.cpu().numpy(), S) and np.array_equal(dl.qserve_s2_zeros.cpu().numpy(), Z)
+    assert np.array_equal(dl.qserve_s1_scales.cpu().numpy().view(np.uint16), s1.reshape(-1).view(np.uint16))
+    prep = O.prepare_weights(w)
+    b = lin.bias.detach().cpu().numpy() if bias else None
+    outs = {}
+    for M in (5, 150):
+        x = O.synth_acts(M, K, seed=M)
+        xd = torch.from_numpy(x).cuda()[None]
+        a8, sx = O.quant_act_i8(x)
+        ref = O.gemm_w4a8_int(a8, prep["qweight"], S, Z, s1.reshape(-1), sx)[1]
+        if b is not None:
+            ref = (ref.astype(np.float32) + b.astype(np.float32)).astype(np.float16)
+        out = dl._forward(xd, M, COMP_TYPE_NAME['w4a8_qserve'])
+        assert np.array_equal(out[0].cpu().numpy().view(np.uint16), ref.view(np.uint16))
+        outs[M] = (xd, out.clone())
+        # nibbles of one quantiser, factors of another (as in the reference): only roughly the fp16 product -- a sanity
+        # bound that a wrong table or a swapped operand would break, not a parity claim
+        assert O.max_abs_rel(out[0].cpu().numpy(), O.switched_forward(x, prep, COMP_TYPE_NAME['fp16'], bias=b)) < 0.3
+        for cid in (COMP_TYPE_NAME['w8a8'], COMP_TYPE_NAME['w4a16_gemm']):
+            assert torch.equal(dl._forward(xd, M, cid), plain._forward(xd, M, cid))
+    assert set(dl.state_dict()) - set(plain.state_dict()) == {"qserve_s1_scales", "qserve_s2_scales", "qserve_s2_zeros"}
+    path = tmp_path / "v2.pt"
+    torch.save(dl.state_dict(), path)
+    fresh = DynamicLinear(K, N, bias, 'cuda', 128)                # the plain constructor: shapes come from the file
+    fresh.load_state_dict(torch.load(path, weights_only=True))
+    for M, (xd, ref) in outs.items():
+        assert torch.equal(fresh._forward(xd, M, COMP_TYPE_NAME['w4a8_qserve']), ref)
+
+
 @pytest.mark.parametrize("cls_name", ["DynamicLinear", "SwitchLinear"])
 def test_checkpoint_round_trip_keeps_every_lane(gpu, cls_name, tmp_path):
     """Dump a quantised layer, load it into an init_only module (on the CPU, then moved to the GPU, as
