@@ -104,3 +104,26 @@ def test_host_mirror_equals_oracle():
     q4, c2 = W.qserve_quantize_tensor_int4(q8, group_size=128)
     assert np.array_equal(q8.numpy(), w8) and np.array_equal(q4.numpy(), q)
     assert c2["scale"].dtype == torch.int8 and c2["zero_pt"].dtype == torch.int8
+
+
+def test_version2_layer_keeps_the_integer_factors_on_the_host():
+    """Host logic of from_module(..., qserve_factors=True): three more buffers beside the six resident ones, carried by
+    the state dict into a module built with the plain constructor; without a GPU the lane itself refuses loudly."""
+    from kairos.dynamic_linear_v2 import COMP_TYPE_NAME, DynamicLinear
+    lin = torch.nn.Linear(256, 64, bias=True, dtype=torch.float16)
+    plain = DynamicLinear.from_module(lin, 'cpu')
+    q = DynamicLinear.from_module(lin, 'cpu', qserve_factors=True)
+    extra = {"qserve_s1_scales", "qserve_s2_scales", "qserve_s2_zeros"}
+    assert set(q.state_dict()) - set(plain.state_dict()) == extra and plain.qserve_s2_scales is None
+    w8, s1 = O.qserve_quantize_int8(lin.weight.detach().numpy())
+    _, si, zi = O.qserve_quantize_int4(w8)
+    S, Z = O.qserve_tables(si, zi, 64)
+    assert np.array_equal(q.qserve_s2_scales.numpy(), S) and np.array_equal(q.qserve_s2_zeros.numpy(), Z)
+    fresh = DynamicLinear(256, 64, True, 'cpu', 128)
+    fresh.load_state_dict(q.state_dict())
+    for key in extra:
+        assert torch.equal(getattr(fresh, key), getattr(q, key))
+    empty = DynamicLinear.from_module(lin, 'cpu', init_only=True, qserve_factors=True)
+    assert empty.qserve_s2_zeros.shape == (2, 64) and empty.qserve_s1_scales.dtype == torch.float16
+    with pytest.raises(ValueError, match="GPU tensor"):
+        q._forward(torch.zeros(1, 3, 256, dtype=torch.float16), 3, COMP_TYPE_NAME['w4a8_qserve'])
