@@ -325,6 +325,19 @@ int kmi_probe_empty(void* stream);
 int kmi_probe_stream_read(const void* buf, size_t bytes, void* stream);
 int kmi_probe_gemv_read(const void* qweight, int N, int K, int nt, int nw, void* stream);
 
+/* Register-only probes of the matrix and vector pipes (no counterpart in the reference either).
+ * kmi_probe_mfma_stream: `workgroups` x 4 waves each issue iters x 16 independent MFMAs (kind 0: v_mfma_i32_32x32x32_i8,
+ * 1: v_mfma_f32_32x32x16_f16) on the 32 KiB of operands at `operands` (device; their bit pattern decides the power drawn);
+ * clocks_u64x2 (device) receives the shader cycles and the ticks of the constant 100 MHz counter around the loop of
+ * workgroup 0, so cycles / ticks * 100 is the shader clock in MHz under that load.
+ * kmi_probe_pipe_overlap: one workgroup of eight waves (two per SIMD), 2048 int8 MFMAs and / or 16384 vector instructions
+ * per wave; cycles_u64x8 (device) receives each wave's cycles.  mode 1: waves 0-3 MFMAs only; 2: waves 4-7 vector
+ * instructions only; 3: both; 4..8: waves 0-3 with 0, 4, 8, 12, 16 vector instructions behind every MFMA; 9: all waves
+ * vector only; 10: waves 0-3 MFMA + 16, waves 4-7 MFMAs only; 11: all waves MFMA + 8; 12: all waves MFMAs only. */
+int kmi_probe_mfma_stream(int kind, const void* operands, size_t operand_bytes, int workgroups, int iters,
+                          void* clocks_u64x2, void* stream);
+int kmi_probe_pipe_overlap(int mode, void* cycles_u64x8, void* stream);
+
 /* ---- bounded conversion buffer (host only) ------------------------------------------------------ */
 
 /* The lanes that convert on demand (W8A8, fp16, W8A16) write the converted weight into a temporary buffer; the

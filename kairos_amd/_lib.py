@@ -64,6 +64,8 @@ SIGNATURES = {
     "kmi_probe_empty": [_P],
     "kmi_probe_stream_read": [_P, _Z, _P],
     "kmi_probe_gemv_read": [_P, _I, _I, _I, _I, _P],
+    "kmi_probe_mfma_stream": [_I, _P, _Z, _I, _I, _P, _P],
+    "kmi_probe_pipe_overlap": [_I, _P, _P],
     "kmi_cache_create": [_P, _Z],
     "kmi_cache_destroy": [_P],
     "kmi_cache_acquire": [_P, ctypes.c_uint64, _I, _Z, ctypes.POINTER(_P)],

@@ -6,6 +6,8 @@
     python -m kairos_amd.bench_extra blasref   # the library's int8 / fp16 GEMMs of this image (hipBLASLt via torch) beside this build's
     python -m kairos_amd.bench_extra weightprep  # offline fp16 -> resident int4 format (device kernel vs host chain), W4A8 re-pack
     python -m kairos_amd.bench_extra actnorm   # per-token quantiser and fused residual add + RMSNorm + quantiser, GB/s
+    python -m kairos_amd.bench_extra floor     # empty launch, plain reader, own-loads reader beside the small-M kernel
+    python -m kairos_amd.bench_extra pipes     # MFMA rate and clock under the power limit, matrix / vector pipe overlap, GEMM by operand activity
 
 Each prints one JSON document.  Inputs are synthetic (N(0, 0.02) weights, N(0, 1) activations with 1 % of the
 channels scaled x20); timing uses device events around back-to-back calls after warm-up, with weight copies rotated
@@ -163,6 +165,83 @@ def floor(args):
         print(row, file=sys.stderr, flush=True)
         del qw
         torch.cuda.empty_cache()
+    return out
+
+
+PIPE_MODES = {1: "waves 0-3: MFMAs only", 2: "waves 4-7: vector instructions only", 3: "both at once, one wave of each kind per SIMD",
+              4: "one wave per SIMD: MFMA + 0 vector instructions", 5: "one wave per SIMD: MFMA + 4", 6: "one wave per SIMD: MFMA + 8",
+              7: "one wave per SIMD: MFMA + 12", 8: "one wave per SIMD: MFMA + 16", 9: "two vector-only waves per SIMD",
+              10: "wave A: MFMA + 16, wave B: MFMAs only", 11: "both waves: MFMA + 8", 12: "two MFMA-only waves per SIMD"}
+
+
+def pipes(args):
+    """What the matrix pipes sustain under the chip's power limit, and how the matrix and vector pipes of a SIMD share one
+    wave or two.  (1) Register-only MFMA loops on 1024 workgroups (no memory traffic), constant against random operands:
+    sustained rate and shader clock.  (2) One workgroup of eight waves, 2048 int8 MFMAs and / or 16384 v_perm_b32 per wave:
+    cycles by mix.  (3) The W8A8 GEMM of the headline (4096 x 28672 x 4096, 256 x 256 tiles) on operands of different bit
+    activity: same kernel and schedule, other power."""
+    from . import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    st = ops._stream()
+    out = {"bench": "pipes", "mfma_stream": [], "overlap": [], "gemm_by_operand_activity": []}
+    wgs, iters = 1024, args.iters
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    for kind, name, ops_per in ((0, "v_mfma_i32_32x32x32_i8", 65536.0), (1, "v_mfma_f32_32x32x16_f16", 32768.0)):
+        for operands in ("constant", "random"):
+            if kind == 0:
+                buf = (torch.full((8192,), 0x01010101, dtype=torch.int32) if operands == "constant"
+                       else torch.randint(-2 ** 31, 2 ** 31 - 1, (8192,), dtype=torch.int32, generator=gen))
+            else:       # fp16: 1.0, or values of magnitude 0.125..0.5 with random mantissas and signs
+                buf = (torch.ones(16384, dtype=torch.float16) if operands == "constant"
+                       else ((torch.rand(16384, generator=gen) * 0.375 + 0.125) * (torch.randint(0, 2, (16384,), generator=gen) * 2 - 1)).to(torch.float16))
+            buf = buf.to(dev)
+            best = None
+            for _ in range(3):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                _lib.check(lib.kmi_probe_mfma_stream(kind, buf.data_ptr(), buf.numel() * buf.element_size(), wgs, iters, clk.data_ptr(), st))
+                b.record()
+                torch.cuda.synchronize()
+                ms = a.elapsed_time(b)
+                c = clk.tolist()
+                if best is None or ms < best[0]:
+                    best = (ms, c)
+            ms, c = best
+            tops = wgs * 4 * iters * 16 * ops_per / (ms * 1e-3) / 1e12
+            row = {"instruction": name, "operands": operands, "ms": round(ms, 2), "tops": round(tops, 1),
+                   "frac_of_published_peak": round(tops / (5000.0 if kind == 0 else 2500.0), 3),
+                   "shader_mhz": round(c[0] / max(c[1], 1) * 100.0), "cycles_per_mfma_and_wave": round(c[0] / (iters * 16.0), 2)}
+            out["mfma_stream"].append(row)
+            print(row, file=sys.stderr, flush=True)
+    cyc = torch.zeros(8, dtype=torch.int64, device=dev)
+    for mode, what in PIPE_MODES.items():
+        for _ in range(2):
+            cyc.zero_()
+            _lib.check(lib.kmi_probe_pipe_overlap(mode, cyc.data_ptr(), st))
+            torch.cuda.synchronize()
+        c = cyc.tolist()
+        row = {"mode": mode, "what": what, "cycles_wave0": c[0], "cycles_wave4": c[4]}
+        out["overlap"].append(row)
+        print(row, file=sys.stderr, flush=True)
+    M, N, K = 4096, 28672, 4096
+    # tiled weights: for zeros and independent random bytes the layout does not matter
+    weights = {"zeros": torch.zeros((N, K), device=dev, dtype=torch.int8),
+               "small": torch.randint(-3, 4, (N, K), device=dev, dtype=torch.int8),
+               "random": torch.randint(-128, 128, (N, K), device=dev, dtype=torch.int8)}
+    acts = {"zeros": torch.zeros((M, K), device=dev, dtype=torch.int8),
+            "small": torch.randint(-3, 4, (M, K), device=dev, dtype=torch.int8),
+            "random": torch.randint(-128, 128, (M, K), device=dev, dtype=torch.int8)}
+    ws = torch.rand(N, device=dev, dtype=torch.float16)
+    asc = torch.rand(M, device=dev, dtype=torch.float16)
+    y = torch.empty((M, N), device=dev, dtype=torch.float16)
+    for an, wn in (("zeros", "zeros"), ("zeros", "random"), ("small", "small"), ("small", "random"), ("random", "random")):
+        us = _time(lambda i: ops.w8a8_gemm_forward(acts[an], weights[wn], ws, asc, y, tiled=True), 20)
+        row = {"M": M, "N": N, "K": K, "activations": an, "weights": wn, "us": round(us, 1),
+               "tops": round(2.0 * M * N * K / us / 1e6, 1), "frac_of_published_peak": round(2.0 * M * N * K / us / 1e-6 / 5.0e15, 3)}
+        out["gemm_by_operand_activity"].append(row)
+        print(row, file=sys.stderr, flush=True)
     return out
 
 
@@ -632,6 +711,8 @@ def main(argv=None):
     sub = ap.add_subparsers(dest="cmd", required=True)
     sub.add_parser("gemv70b")
     sub.add_parser("floor")
+    pp = sub.add_parser("pipes")
+    pp.add_argument("--iters", type=int, default=200000, help="16-MFMA rounds per wave of the chip-wide loop (200000: ~0.2 s per run)")
     sub.add_parser("convert")
     sub.add_parser("weightprep")
     sub.add_parser("blasref")
@@ -652,7 +733,7 @@ def main(argv=None):
     if args.cmd == "decoder" and args.lut is None:
         import os
         args.lut = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prof", "llama3_8b_mi355x_v2") + "/"
-    res = {"gemv70b": gemv70b, "floor": floor, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
+    res = {"gemv70b": gemv70b, "floor": floor, "pipes": pipes, "convert": convert, "weightprep": weightprep, "blasref": blasref, "actnorm": actnorm, "decoder": decoder}[args.cmd](args)
     print(json.dumps(res))
 
 

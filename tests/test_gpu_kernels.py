@@ -1101,3 +1101,35 @@ def test_random_shapes_every_variant_agrees(ops):
             assert (o.float() - want).abs().max().item() / scale < 4e-3, (tag, "small-M kernel")
         o = ops.f16_gemm_forward(x, w16, N, bias=bias)
         assert (o.float() - want).abs().max().item() / scale < 4e-3, (tag, "fp16 GEMM")
+
+
+def test_pipe_probes_measure_what_they_say():
+    """The register-only probes behind the pipe figures: a lone wave's int8 32 x 32 x 32 MFMA holds the matrix pipe 32
+    cycles (8 passes of 4), a few vector instructions behind each MFMA are free and many are not, a vector-only wave
+    runs beside an MFMA-only wave of the same SIMD in far less than the sum of their times, and the chip-wide loop
+    reports a plausible clock."""
+    import kairos_amd._lib as L
+    lib = L.load()
+    cyc = torch.zeros(8, dtype=torch.int64, device="cuda")
+
+    def run(mode):
+        for _ in range(2):
+            L.check(lib.kmi_probe_pipe_overlap(mode, cyc.data_ptr(), None))
+            torch.cuda.synchronize()
+        return cyc.tolist()
+    alone = run(1)[0]
+    valu = run(2)[4]
+    both = run(3)
+    assert 30.0 < alone / 2048 < 40.0
+    assert 3.5 < valu / 16384 < 8.0
+    assert both[0] < 1.15 * alone and both[4] < 0.85 * (alone + valu)
+    assert run(5)[0] < 1.15 * alone and run(8)[0] > 1.8 * alone          # + 4 hidden, + 16 not
+    with pytest.raises(RuntimeError):
+        L.check(lib.kmi_probe_pipe_overlap(13, cyc.data_ptr(), None))
+    clk = torch.zeros(2, dtype=torch.int64, device="cuda")
+    buf = torch.full((8192,), 0x01010101, dtype=torch.int32, device="cuda")
+    L.check(lib.kmi_probe_mfma_stream(0, buf.data_ptr(), buf.numel() * 4, 256, 2000, clk.data_ptr(), None))
+    torch.cuda.synchronize()
+    c = clk.tolist()
+    assert 30.0 < c[0] / (2000 * 16) < 40.0                              # one wave per SIMD: back-to-back MFMAs
+    assert 800 < c[0] / c[1] * 100 < 2600                                 # MHz
