@@ -179,7 +179,8 @@ def pipes(args):
     wave or two.  (1) Register-only MFMA loops on 1024 workgroups (no memory traffic), constant against random operands:
     sustained rate and shader clock.  (2) One workgroup of eight waves, 2048 int8 MFMAs and / or 16384 v_perm_b32 per wave:
     cycles by mix.  (3) The W8A8 GEMM of the headline (4096 x 28672 x 4096, 256 x 256 tiles) on operands of different bit
-    activity: same kernel and schedule, other power."""
+    activity: same kernel and schedule, other power.  (4) That kernel's time per k-stage with 1, 64 and 256 tiles in
+    flight: what the schedule costs alone and what the clock takes when every CU multiplies random bytes."""
     from . import _lib
     lib = _lib.load()
     dev = torch.device("cuda:0")
@@ -242,6 +243,34 @@ def pipes(args):
                "tops": round(2.0 * M * N * K / us / 1e6, 1), "frac_of_published_peak": round(2.0 * M * N * K / us / 1e-6 / 5.0e15, 3)}
         out["gemm_by_operand_activity"].append(row)
         print(row, file=sys.stderr, flush=True)
+    # (4) the same kernel's time per 64-byte k-stage (32 MFMAs of 32 cycles per wave = 1024 cycles = 427 ns at 2.4 GHz)
+    # from two K at a fixed number of 256 x 256 tiles: a lone workgroup, a quarter of the chip, every CU
+    del weights, acts
+    out["w8a8_stage_time"] = []
+    for data in ("zeros", "random"):
+        for M, N in ((256, 256), (2048, 2048), (4096, 4096)):
+            us = {}
+            for K in (8192, 32768):
+                if data == "zeros":
+                    a8 = torch.zeros((M, K), device=dev, dtype=torch.int8)
+                    w8 = torch.zeros((N, K), device=dev, dtype=torch.int8)
+                else:
+                    a8 = torch.randint(-128, 128, (M, K), device=dev, dtype=torch.int8)
+                    w8 = torch.randint(-128, 128, (N, K), device=dev, dtype=torch.int8)
+                ws, asc = torch.rand(N, device=dev, dtype=torch.float16), torch.rand(M, device=dev, dtype=torch.float16)
+                y = torch.empty((M, N), device=dev, dtype=torch.float16)
+                ops.force_gemm_tile(256)
+                ops.force_gemm_splits(1)
+                try:
+                    us[K] = min(_time(lambda i: ops.w8a8_gemm_forward(a8, w8, ws, asc, y, tiled=True), 20) for _ in range(3))
+                finally:
+                    ops.force_gemm_tile(0)
+                    ops.force_gemm_splits(0)
+            ns = (us[32768] - us[8192]) * 1e3 / ((32768 - 8192) / 64)
+            row = {"operands": data, "tiles": (M // 256) * (N // 256), "us_k8192": round(us[8192], 1), "us_k32768": round(us[32768], 1),
+                   "ns_per_stage": round(ns), "mfma_cycles_over_time_ghz": round(1024.0 / ns, 2)}
+            out["w8a8_stage_time"].append(row)
+            print(row, file=sys.stderr, flush=True)
     return out
 
 
